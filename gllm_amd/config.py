@@ -63,6 +63,10 @@ class EngineConfig:
     enable_prefix_caching: bool = True
     kv_cache_dtype: str = "auto"         # "auto" | "fp8"
 
+    # recurrent-state slots for hybrid models (one per live sequence);
+    # None = maxd + 64. A small value makes slots recycle under test.
+    max_state_slots: Optional[int] = None
+
     # --- scheduler ---
     schedule_method: str = "token_throttling"  # chunked_prefill|token_throttling|split_pd
     maxp: int = 8192                     # max prefill tokens per tick

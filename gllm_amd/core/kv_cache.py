@@ -34,13 +34,27 @@ class KVCacheSpec:
     # absorbed MLA: the v-cache is a zero-copy view of the latent
     # k-cache's first v_head_dim dims — only k bytes are allocated
     v_shared: bool = False
+    # heterogeneous stacks: (kv_heads, k_dim, v_dim) per cache-owning
+    # layer; when set, num_layers/num_kv_heads/head_dim/v_head_dim above
+    # describe layer 0 only and every layer's cache has its own shape
+    layer_shapes: Optional[List[Tuple[int, int, int]]] = None
 
     def __post_init__(self):
         if not self.v_head_dim:
             self.v_head_dim = self.head_dim
 
+    def shapes(self) -> List[Tuple[int, int, int]]:
+        if self.layer_shapes is not None:
+            return list(self.layer_shapes)
+        return [(self.num_kv_heads, self.head_dim, self.v_head_dim)
+                ] * self.num_layers
+
     @property
     def bytes_per_page(self) -> int:
+        if self.layer_shapes is not None:
+            return max(1, sum(self.page_size * g * (dk + dv)
+                              * self.dtype_bytes
+                              for g, dk, dv in self.layer_shapes))
         v = 0 if self.v_shared else self.v_head_dim
         return (self.num_layers * self.page_size * self.num_kv_heads
                 * (self.head_dim + v) * self.dtype_bytes)

@@ -385,6 +385,66 @@ class Scheduler:
         return decode_batch + prefill_batch
 
     # ------------------------------------------------------------------
+    # scripted mode: the caller dictates the batch (trace replay, scoring
+    # of given continuations). Same ScheduledBatch records, page
+    # allocation and in-flight bookkeeping as the policies above; the
+    # sequences never enter the prefill/decode queues.
+    # ------------------------------------------------------------------
+    def schedule_scripted(self, chunks) -> Optional[ScheduledBatch]:
+        """``chunks``: [(seq, n)] — advance ``seq`` by its next ``n``
+        tokens (already present in seq.token_ids). One batch, in the
+        given order; raises MemoryError when the page pool cannot hold
+        it (nothing is allocated then)."""
+        if len(self.batch_running) >= self.pp_size:
+            return None
+        plan = []
+        need_total = 0
+        for seq, n in chunks:
+            start = self._sched_cursor(seq)
+            if n <= 0 or start + n > len(seq.token_ids):
+                raise ValueError(
+                    f"seq {seq.seq_id}: cannot advance {n} tokens from "
+                    f"{start} (holds {len(seq.token_ids)})")
+            pages_total = -(-(start + n) // self.page_size)
+            need = max(0, pages_total - len(seq.page_table))
+            plan.append((seq, start, n, need))
+            need_total += need
+        if need_total > self.mm.get_num_free_pages():
+            raise MemoryError(
+                f"scripted batch needs {need_total} pages, "
+                f"{self.mm.get_num_free_pages()} free")
+        items = []
+        for seq, start, n, need in plan:
+            if need:
+                seq.page_table.extend(self.mm._allocate_fresh(need))
+            items.append(ScheduledSeq(seq, start, n))
+            self._scheduled_cursor[seq.seq_id] = start + n
+        if not items:
+            return None
+        self._batch_counter += 1
+        batch = ScheduledBatch(items, self._batch_counter)
+        self.batch_running.append(batch)
+        return batch
+
+    def commit_scripted(self, batch: ScheduledBatch) -> None:
+        """Commit a scripted batch's cursors (no token is appended)."""
+        assert self.batch_running and self.batch_running[0] is batch, \
+            "batches must commit in FIFO order"
+        self.batch_running.popleft()
+        for item in batch.items:
+            seq = item.seq
+            seq.computed_token_num = item.start + item.num_tokens
+            if isinstance(self.mm, PrefixMemoryManager):
+                self.mm.register_computed_pages(seq)
+
+    def release_scripted(self, seq: Sequence) -> None:
+        """Give back everything a scripted sequence holds (KV pages,
+        state slot, penalty slot) so later requests re-use it."""
+        assert not self._in_flight(seq)
+        self.mm.free_seq(seq)
+        self._scheduled_cursor.pop(seq.seq_id, None)
+
+    # ------------------------------------------------------------------
     # output processing
     # ------------------------------------------------------------------
     def process_output(self, batch: ScheduledBatch,

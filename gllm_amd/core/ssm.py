@@ -13,6 +13,7 @@ manager's hit_filter trims hits to the deepest snapshotted boundary.
 
 import collections
 import dataclasses
+from typing import List, Optional
 
 import torch
 
@@ -28,6 +29,22 @@ class SSMSpec:
     num_v_heads: int     # per TP rank
     head_k_dim: int
     head_v_dim: int
+    # heterogeneous stacks: one SSMLayerSpec per recurrent layer (the
+    # uniform fields above are then ignored). Each layer gets its own
+    # conv/recurrent tensors, so layers may differ in every size.
+    layers: Optional[List["SSMLayerSpec"]] = None
+
+
+@dataclasses.dataclass
+class SSMLayerSpec:
+    conv_dim: int
+    conv_kernel: int
+    num_v_heads: int
+    head_k_dim: int
+    head_v_dim: int
+    # recurrent state [H, Dk, Dv] ("kv": the delta-rule kernels that keep
+    # a value-column block per wavefront) or [H, Dv, Dk] ("vk")
+    layout: str = "kv"
 
 
 class SSMPool:
@@ -36,12 +53,24 @@ class SSMPool:
         self.spec = spec
         self.device = device
         L = spec.num_ssm_layers
-        self.conv_state = torch.zeros(
-            L, num_slots, spec.conv_dim, spec.conv_kernel - 1,
-            dtype=dtype, device=device)
-        self.ssm_state = torch.zeros(
-            L, num_slots, spec.num_v_heads, spec.head_v_dim,
-            spec.head_k_dim, dtype=torch.float32, device=device)
+        if spec.layers is not None:
+            # per-layer geometry: lists indexed by ssm layer id (the
+            # uniform case below is one stacked tensor, indexed alike)
+            self.conv_state = [torch.zeros(
+                num_slots, ls.conv_dim, max(ls.conv_kernel - 1, 1),
+                dtype=dtype, device=device) for ls in spec.layers]
+            self.ssm_state = [torch.zeros(
+                (num_slots, ls.num_v_heads) + (
+                    (ls.head_k_dim, ls.head_v_dim) if ls.layout == "kv"
+                    else (ls.head_v_dim, ls.head_k_dim)),
+                dtype=torch.float32, device=device) for ls in spec.layers]
+        else:
+            self.conv_state = torch.zeros(
+                L, num_slots, spec.conv_dim, spec.conv_kernel - 1,
+                dtype=dtype, device=device)
+            self.ssm_state = torch.zeros(
+                L, num_slots, spec.num_v_heads, spec.head_v_dim,
+                spec.head_k_dim, dtype=torch.float32, device=device)
         # the LAST slot is the hipGraph dummy/scratch slot (padding rows
         # of a captured decode bucket write their garbage there); the
         # allocator never hands it out
@@ -76,8 +105,12 @@ class SSMPool:
 
     def snapshot(self, chain_id: int, slot: int) -> None:
         snaps = self.snapshots
-        snaps[chain_id] = (self.conv_state[:, slot].clone(),
-                           self.ssm_state[:, slot].clone())
+        if isinstance(self.conv_state, list):
+            snaps[chain_id] = ([c[slot].clone() for c in self.conv_state],
+                               [r[slot].clone() for r in self.ssm_state])
+        else:
+            snaps[chain_id] = (self.conv_state[:, slot].clone(),
+                               self.ssm_state[:, slot].clone())
         snaps.move_to_end(chain_id)
         while len(snaps) > self.max_snapshots:
             snaps.popitem(last=False)
@@ -87,6 +120,12 @@ class SSMPool:
         if snap is None:
             return False
         self.snapshots.move_to_end(chain_id)
-        self.conv_state[:, slot].copy_(snap[0])
-        self.ssm_state[:, slot].copy_(snap[1])
+        if isinstance(self.conv_state, list):
+            for c, sc in zip(self.conv_state, snap[0]):
+                c[slot].copy_(sc)
+            for r, sr in zip(self.ssm_state, snap[1]):
+                r[slot].copy_(sr)
+        else:
+            self.conv_state[:, slot].copy_(snap[0])
+            self.ssm_state[:, slot].copy_(snap[1])
         return True

@@ -6,6 +6,7 @@ kernel family (prefill MFMA kernel / split-KV decode kernel, dispatched
 in ops.paged_attention).
 """
 
+from typing import Optional
 
 import torch
 import torch.nn as nn
@@ -45,3 +46,85 @@ class Attention(nn.Module):
             max_query_len=fctx.max_query_len,
             sliding_window=self.sliding_window)
         return out.reshape(T, -1)
+
+
+class WindowAttention(nn.Module):
+    """Paged attention with a sliding window that keeps the first tokens
+    visible, an optional softmax sink and a fused output gate.
+
+    * per-head query/key size ``head_dim`` and value size ``v_head_dim``
+      may differ; any GQA ratio
+    * q/k get a per-head RMS norm (plain weights ``q_norm``/``k_norm``)
+      and an interleaved-pair rotary (``rotary``: layers.rotary
+      .PairRotary or None) inside one fused kernel that also stores k, v
+      in the paged cache
+    * position i sees j <= i with i - j < ``window`` or j < ``keep_first``
+      (window 0 = plain causal)
+    * ``sink``: softmax denominator 1 + sum exp(s)
+    * ``kv_source``: cache index of ANOTHER layer whose keys and values
+      this layer attends over; such a layer owns no k/v tensors and
+      stores nothing (``owns_kv`` False)
+
+    Everything runs in the dtype of q (bf16 or fp32) with fp32 scores.
+    """
+
+    def __init__(self, layer_idx: int, num_heads: int, num_kv_heads: int,
+                 head_dim: int, v_head_dim: int, scale: float, eps: float,
+                 window: int = 0, keep_first: int = 0, sink: bool = False,
+                 rotary: Optional[nn.Module] = None, owns_kv: bool = True,
+                 params_dtype=None):
+        super().__init__()
+        dtype = params_dtype or torch.get_default_dtype()
+        self.layer_idx = layer_idx       # cache this layer reads
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.v_head_dim = v_head_dim
+        self.scale = scale
+        self.eps = eps
+        self.window = window
+        self.keep_first = keep_first
+        self.sink = sink
+        self.rotary = rotary
+        self.owns_kv = owns_kv
+        self.q_norm = nn.Parameter(torch.ones(head_dim, dtype=dtype),
+                                   requires_grad=False)
+        if owns_kv:
+            self.k_norm = nn.Parameter(torch.ones(head_dim, dtype=dtype),
+                                       requires_grad=False)
+        self._no_rot = None
+
+    def _freqs(self, device):
+        if self.rotary is not None:
+            return self.rotary.freqs, self.rotary.mag, self.rotary.rot_dims
+        if self._no_rot is None or self._no_rot.device != device:
+            self._no_rot = torch.zeros(1, dtype=torch.float64, device=device)
+        return self._no_rot, 1.0, 0
+
+    def forward(self, q: torch.Tensor, k: Optional[torch.Tensor],
+                v: Optional[torch.Tensor], gate: Optional[torch.Tensor],
+                fctx: ForwardContext) -> torch.Tensor:
+        """q [T, H*D], k [T, G*D], v [T, G*Dv], gate [T, H*Dv] (row
+        views of a merged projection are fine). Returns [T, H*Dv]."""
+        T = q.shape[0]
+        if fctx.is_profile_run:
+            return q.new_zeros(T, self.num_heads * self.v_head_dim)
+        k_cache = fctx.k_caches[self.layer_idx]
+        v_cache = fctx.v_caches[self.layer_idx]
+        freqs, mag, rot_dims = self._freqs(q.device)
+        if self.owns_kv:
+            ops.qk_norm_rope_store(
+                q, k, v, self.q_norm, self.k_norm, fctx.positions,
+                fctx.slot_mapping, freqs, mag, rot_dims, k_cache, v_cache,
+                self.num_heads, self.num_kv_heads, self.head_dim,
+                self.v_head_dim, self.eps)
+        else:
+            ops.qk_norm_rope_store(
+                q, None, None, self.q_norm, None, fctx.positions,
+                fctx.slot_mapping, freqs, mag, rot_dims, None, None,
+                self.num_heads, self.num_kv_heads, self.head_dim,
+                self.v_head_dim, self.eps)
+        return ops.window_attention(
+            q, gate, k_cache, v_cache, fctx.block_table, fctx.seq_lens,
+            fctx.query_start_loc, self.scale, self.window,
+            self.keep_first, self.sink)

@@ -44,3 +44,39 @@ class GemmaRMSNorm(nn.Module):
             return ops.fused_add_rmsnorm(x, residual, self._scale(),
                                          self.eps)
         return ops.rmsnorm(x, self._scale(), self.eps)
+
+
+class LayerNorm(nn.Module):
+    """LayerNorm with weight and bias over an fp32 residual stream.
+
+    Sandwich-norm decoders (a norm before and after every sublayer) keep
+    the stream in fp32 while sublayers run in the model dtype:
+
+    * ``norm(x)``                       h = LN(x), x fp32 -> model dtype
+    * ``norm.add_into(x, y, nxt)``      x += LN(y) in place and, when
+      ``nxt`` (the next sublayer's pre-norm) is given, returns nxt(x) —
+      one fused launch per boundary (ops.residual_layernorm)
+
+    The bias parameter is named ``bias``; checkpoints that store it
+    under another name map it in the model's load_weights.
+    """
+
+    def __init__(self, hidden_size: int, eps: float = 1e-5,
+                 params_dtype=None):
+        super().__init__()
+        dtype = params_dtype or torch.get_default_dtype()
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype),
+                                   requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=dtype),
+                                 requires_grad=False)
+        self.eps = eps
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.layernorm_f32(x, self.weight, self.bias, self.eps,
+                                 self.weight.dtype)
+
+    def add_into(self, x: torch.Tensor, y: torch.Tensor,
+                 nxt: Optional["LayerNorm"] = None):
+        pre = (nxt.weight, nxt.bias) if nxt is not None else None
+        return ops.residual_layernorm(x, y, self.weight, self.bias,
+                                      self.eps, pre)

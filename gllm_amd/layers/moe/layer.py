@@ -130,7 +130,8 @@ class FusedMoE(nn.Module):
         ``sel.any()`` form synced once per expert: 256/layer on
         DeepSeek-V3). DP padding rows carry expert id -1 and land in
         segment 0 of the shifted bincount (skipped)."""
-        if (x.is_cuda and x.dtype == torch.bfloat16 and ops.has_kernels()):
+        if (x.is_cuda and x.dtype == torch.bfloat16
+                and ops.has_moe_kernels()):
             if self.int4_packed is not None:
                 # compressed-tensors int4 experts (Kimi-K2.5): run the
                 # bf16 grouped MFMA GEMM over a one-time dequantized
@@ -152,7 +153,11 @@ class FusedMoE(nn.Module):
                     x.contiguous(), w13s, w2s, weights, ids,
                     expert_start=self.expert_start,
                     num_global_experts=self.num_experts)
-            if self.fp8_block is None and self.int4_cfg is None:
+            if (self.fp8_block is None and self.int4_cfg is None
+                    and x.shape[1] % 8 == 0
+                    and self.intermediate_per_rank % 8 == 0):
+                # (the grouped GEMM loads 8-element bf16 vectors along
+                # K; odd widths take the segment loop below)
                 return ops.fused_moe(
                     x.contiguous(), self.w13_weight, self.w2_weight,
                     weights, ids, expert_start=self.expert_start,

@@ -193,3 +193,44 @@ def get_rope(head_dim: int, rot_dim: int, max_position: int, base: float,
             raise ValueError(f"unsupported rope_type {rtype}")
     _ROPE_CACHE[key] = rope
     return rope
+
+
+class PairRotary(nn.Module):
+    """Interleaved-pair rotary table: dimension 2i rotates with 2i+1 on
+    the first ``rot_dims`` dims of a head, the rest pass through.
+
+    Holds only the per-pair frequencies (fp64) and the cos/sin
+    magnitude; angles are formed inside the fused q/k kernel
+    (ops.qk_norm_rope_store) as position * frequency in fp64, so there is
+    no max-position table to size. ``scaling`` = dict(factor, original,
+    fast, slow) applies YaRN: pairs whose wavelength exceeds the original
+    context (ramp 1) are slowed by ``factor``, short-wavelength pairs
+    (ramp 0) keep their frequency, with a linear ramp between the
+    correction dims of ``fast`` and ``slow`` rotations, and cos/sin are
+    scaled by 0.1 ln(factor) + 1.
+    """
+
+    def __init__(self, rot_dims: int, base: float,
+                 scaling: Optional[dict] = None):
+        super().__init__()
+        assert rot_dims % 2 == 0
+        self.rot_dims = rot_dims
+        i = torch.arange(rot_dims // 2, dtype=torch.float64)
+        freqs = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                          -2.0 * i / max(rot_dims, 1))
+        self.mag = 1.0
+        if scaling:
+            factor = float(scaling["factor"])
+            orig = float(scaling["original"])
+
+            def correction_dim(turns: float) -> float:
+                return rot_dims * math.log(orig / (2 * math.pi * turns)) \
+                    / (2 * math.log(base))
+
+            lo = max(math.floor(correction_dim(float(scaling["fast"]))), 0)
+            hi = min(math.ceil(correction_dim(float(scaling["slow"]))),
+                     rot_dims - 1)
+            ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+            freqs = freqs / factor * ramp + freqs * (1.0 - ramp)
+            self.mag = 0.1 * math.log(factor) + 1.0
+        self.register_buffer("freqs", freqs, persistent=False)

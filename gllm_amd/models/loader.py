@@ -33,7 +33,9 @@ def get_arch_registry():
     from gllm_amd.models.qwen3_vl import (Qwen3VLForCausalLM,
                                           Qwen3VLMoeForCausalLM,
                                           Qwen3_5VLForCausalLM)
+    from gllm_amd.models.sudevik import SudevikForCausalLM
     return {
+        "Sudevik": SudevikForCausalLM,
         "Qwen2VLForConditionalGeneration": Qwen2VLForCausalLM,
         "Qwen2_5_VLForConditionalGeneration": Qwen2VLForCausalLM,
         "Qwen3VLForConditionalGeneration": Qwen3VLForCausalLM,
@@ -201,7 +203,10 @@ def dummy_init(model: torch.nn.Module, seed: int = 0) -> None:
 
 
 def create_model(cfg, engine_config, device: str = "cpu") -> torch.nn.Module:
-    archs = getattr(cfg, "architectures", None) or []
+    archs = list(getattr(cfg, "architectures", None) or [])
+    if isinstance(getattr(cfg, "architecture", None), str):
+        # configs that name ONE architecture under the singular key
+        archs.append(cfg.architecture)
     registry = get_arch_registry()
     cls = None
     for a in archs:

@@ -34,9 +34,49 @@ def _load_kernels():
     return _K
 
 
+_KS = None
+_KS_ERR: Optional[str] = None
+
+
+def _load_seq_kernels():
+    """The dtype-generic sequence-mixer module (setup.py SEQ_SOURCES):
+    built on its own so a model that needs only these kernels serves
+    from a checkout where the full extension was never compiled."""
+    global _KS, _KS_ERR
+    if _KS is not None or _KS_ERR is not None:
+        return _KS
+    try:
+        from gllm_amd import _kernels_seq
+        _KS = _kernels_seq
+    except ImportError as e:  # pragma: no cover
+        _KS_ERR = str(e)
+    return _KS
+
+
+class _SeqBacked:
+    """Stand-in for the full extension when only the sequence-mixer
+    module is built: serves the entry points both modules define (MoE
+    grouped GEMM, gated activations) and fails loudly on the rest."""
+
+    def __init__(self, mod):
+        self._mod = mod
+
+    def __getattr__(self, name):
+        try:
+            return getattr(self._mod, name)
+        except AttributeError:
+            raise RuntimeError(
+                f"kernel {name!r} lives in gllm_amd._kernels, which is "
+                f"not built (import error: {_K_ERR}); run `python "
+                "setup.py build_ext --inplace`") from None
+
+
 def _gpu_kernels():
     k = _load_kernels()
     if k is None:
+        ks = _load_seq_kernels()
+        if ks is not None:
+            return _SeqBacked(ks)
         raise RuntimeError(
             "gllm_amd._kernels HIP extension not built but a CUDA tensor "
             "was passed — build with `python setup.py build_ext --inplace` "
@@ -44,8 +84,23 @@ def _gpu_kernels():
     return k
 
 
+def _seq_kernels():
+    k = _load_seq_kernels()
+    if k is None:
+        raise RuntimeError(
+            "gllm_amd._kernels_seq HIP extension not built but a CUDA "
+            "tensor was passed — build with `GLLM_EXT=seq python setup.py "
+            f"build_ext --inplace`. Import error: {_KS_ERR}")
+    return k
+
+
 def has_kernels() -> bool:
     return _load_kernels() is not None
+
+
+def has_moe_kernels() -> bool:
+    """The bf16 grouped MoE GEMM ships in both extension modules."""
+    return _load_kernels() is not None or _load_seq_kernels() is not None
 
 
 # --------------------------------------------------------------- norm
@@ -134,6 +189,11 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor,
 # --------------------------------------------------------------- moe
 def topk_softmax(gating: torch.Tensor, topk: int, renormalize: bool = True):
     return torch_ref.topk_softmax(gating, topk, renormalize)
+
+
+def topk_then_softmax(logits: torch.Tensor, topk: int):
+    """Top-k over raw router logits, softmax over the chosen only."""
+    return torch_ref.topk_then_softmax(logits, topk)
 
 
 def grouped_topk(scores, topk, n_group, topk_group, renormalize=True,
@@ -673,3 +733,115 @@ def linear(x: torch.Tensor, w: torch.Tensor,
             and _use_skinny(x.shape[0], w.shape[0], w.shape[1])):
         return skinny_gemm(x, w, bias)
     return F.linear(x, w, bias)
+
+
+# --------------------------------------------------------------- layer norm
+def layernorm_f32(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor,
+                  eps: float, dtype) -> torch.Tensor:
+    """h = LayerNorm(x) with weight and bias; x is the fp32 residual
+    stream, h comes out in the model dtype."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=dtype, device=x.device)
+        _seq_kernels().layernorm_f32(out, x, w, b, eps)
+        return out
+    return torch_ref.layernorm_f32(x, w, b, eps, dtype)
+
+
+def residual_layernorm(x: torch.Tensor, y: torch.Tensor, w_post, b_post,
+                       eps: float, pre=None):
+    """x (fp32, in place) += LN_post(y); with ``pre`` = (weight, bias)
+    also returns LN_pre(x) in y's dtype — one launch per layer boundary
+    of a sandwich-norm decoder."""
+    if x.is_cuda:
+        h = None
+        if pre is not None:
+            h = torch.empty(x.shape, dtype=y.dtype, device=x.device)
+            _seq_kernels().residual_layernorm(x, y, w_post, b_post, h,
+                                              pre[0], pre[1], eps)
+        else:
+            _seq_kernels().residual_layernorm(x, y, w_post, b_post, None,
+                                              None, None, eps)
+        return h
+    return torch_ref.residual_layernorm(x, y, w_post, b_post, eps, pre)
+
+
+# --------------------------------------------------------------- windowed attn
+def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
+                       mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps):
+    """Fused per-head q/k RMS norm, interleaved-pair rotary (per-pair
+    frequency table ``freqs`` fp64, cos/sin scaled by ``mag``) and paged
+    K/V store. q [T, H*D] is updated in place (may be a column slice of
+    a merged projection); k/v None = the layer reads another's cache."""
+    if q.is_cuda:
+        _seq_kernels().qk_norm_rope_store(
+            q, k, v, q_w, k_w, positions, slot_mapping, freqs, mag,
+            rot_dims, k_cache, v_cache, H, G, D, Dv, eps)
+        return
+    torch_ref.qk_norm_rope_store(q, k, v, q_w, k_w, positions,
+                                 slot_mapping, freqs, mag, rot_dims,
+                                 k_cache, v_cache, H, G, D, Dv, eps)
+
+
+def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
+                     query_start_loc, scale, window=0, keep_first=0,
+                     sink=False) -> torch.Tensor:
+    """Ragged paged attention over K [pages, page, G, D] / V [.., Dv]:
+    sliding window with kept first tokens, optional softmax sink (+1 in
+    the denominator) and fused sigmoid output gate. Returns [T, H*Dv]."""
+    if q.is_cuda:
+        T = q.shape[0]
+        H = q.shape[1] // k_cache.shape[3]
+        out = torch.empty(T, H * v_cache.shape[3], dtype=q.dtype,
+                          device=q.device)
+        _seq_kernels().window_attention(
+            out, q, gate, k_cache, v_cache, block_table, seq_lens,
+            query_start_loc, scale, window, keep_first, sink)
+        return out
+    return torch_ref.window_attention(q, gate, k_cache, v_cache,
+                                      block_table, seq_lens,
+                                      query_start_loc, scale, window,
+                                      keep_first, sink)
+
+
+# --------------------------------------------------------------- delta rule
+def causal_conv_silu(x, w, conv_state, slots, has_init, query_start_loc):
+    """Ragged short causal conv + silu; rolls ``conv_state`` rows
+    ``slots`` in place. x may be a column slice of a merged projection."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _seq_kernels().causal_conv_silu(out, x, w, conv_state, slots,
+                                        has_init, query_start_loc)
+        return out
+    from gllm_amd.ops import gdn_ref
+    return gdn_ref.causal_conv_silu(x, w, conv_state, slots, has_init,
+                                    query_start_loc)
+
+
+def delta_rule_varlen(q, k, v, a, b, A_log, dt_bias, state, slots,
+                      has_init, query_start_loc, q_scale) -> torch.Tensor:
+    """Ragged gated delta rule (prompt portions and decode tokens in one
+    launch); fp32 state [slots, H, Dk, Dv] in place; returns fp32
+    [T, H, Dv]."""
+    if q.is_cuda:
+        H, _, Dv = state.shape[1:]
+        o = torch.empty(q.shape[0], H, Dv, dtype=torch.float32,
+                        device=q.device)
+        _seq_kernels().delta_rule_varlen(o, q, k, v, a, b, A_log, dt_bias,
+                                         state, slots, has_init,
+                                         query_start_loc, q_scale)
+        return o
+    from gllm_amd.ops import gdn_ref
+    return gdn_ref.delta_rule_varlen(q, k, v, a, b, A_log, dt_bias, state,
+                                     slots, has_init, query_start_loc,
+                                     q_scale)
+
+
+def rms_gate(o, z, w, H, eps, dtype) -> torch.Tensor:
+    """Per head o / rms(o) * w * silu(z): fp32 [T, H, Dv] -> [T, H*Dv]."""
+    if o.is_cuda:
+        out = torch.empty(o.shape[0], o.shape[1] * o.shape[2], dtype=dtype,
+                          device=o.device)
+        _seq_kernels().rms_gate(out, o, z, w, H, eps)
+        return out
+    from gllm_amd.ops import gdn_ref
+    return gdn_ref.rms_gate(o, z, w, H, eps, dtype)

@@ -1,0 +1,349 @@
+// Windowed attention with kept first tokens and a softmax sink, gfx950.
+//
+// Dtype-generic (T = bf16 or fp32 for q/k/v/cache/out; scores, softmax
+// and accumulation are fp32 always) and shape-generic: any per-head
+// query/key size D, value size Dv != D, any GQA ratio, any page size.
+//
+//   qk_norm_rope_store  per-head RMS norm of q and k (plain weight),
+//                       interleaved-pair rotary on the first rot_dims
+//                       dims with a per-pair frequency table (YaRN or
+//                       plain; angle = pos * f in fp64, so long
+//                       positions lose nothing), then q in place and
+//                       k, v scattered into the paged cache
+//   window_attention    ragged batch (prompt portions beside single
+//                       decode tokens) over the paged cache: position i
+//                       sees j <= i with i - j < window or j < keep_first;
+//                       optional sink: softmax denominator 1 + sum exp(s)
+//                       (a score-0 key with no value); optional fused
+//                       sigmoid output gate
+//
+// A layer that shares another layer's keys and values calls
+// qk_norm_rope_store with no k/v and attends over the owner's cache.
+
+#include <torch/extension.h>
+#include <ATen/cuda/CUDAContext.h>
+#include "common.h"
+
+namespace {
+
+constexpr int QK_BLOCK = 64;
+constexpr int ATT_BLOCK = 256;
+
+// ------------------------------------------------------------------
+// grid (tokens, H + 2G): y < H query head (in place), y < H+G key head
+// (norm + rotary -> cache), else value head (plain copy -> cache)
+template <typename T>
+__global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
+    T *__restrict__ q, long q_stride, const T *__restrict__ k, long k_stride,
+    const T *__restrict__ v, long v_stride, const T *__restrict__ q_w,
+    const T *__restrict__ k_w, const long *__restrict__ positions,
+    const long *__restrict__ slot_mapping, const double *__restrict__ freqs,
+    float mag, int rot_dims, T *__restrict__ k_cache, T *__restrict__ v_cache,
+    int H, int G, int D, int Dv, float eps) {
+  extern __shared__ float buf[];
+  const int t = blockIdx.x;
+  const int y = blockIdx.y;
+  const int lane = threadIdx.x;
+  if (y >= H + G) {  // value copy
+    const int g = y - H - G;
+    const long slot = slot_mapping[t];
+    const T *src = v + (long)t * v_stride + (long)g * Dv;
+    T *dst = v_cache + (slot * G + g) * Dv;
+    for (int i = lane; i < Dv; i += QK_BLOCK) dst[i] = src[i];
+    return;
+  }
+  const bool is_q = y < H;
+  const T *src = is_q ? q + (long)t * q_stride + (long)y * D
+                      : k + (long)t * k_stride + (long)(y - H) * D;
+  const T *w = is_q ? q_w : k_w;
+  float ss = 0.f;
+  for (int i = lane; i < D; i += QK_BLOCK) {
+    const float x = ScalarOps<T>::to_f32(src[i]);
+    buf[i] = x;
+    ss += x * x;
+  }
+  ss = wave_reduce_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / D + eps);
+  __syncthreads();
+  for (int i = lane; i < D; i += QK_BLOCK)
+    buf[i] = buf[i] * inv * ScalarOps<T>::to_f32(w[i]);
+  __syncthreads();
+  const double pos = (double)positions[t];
+  for (int p = lane; p < rot_dims / 2; p += QK_BLOCK) {
+    double sn, cs;
+    sincos(pos * freqs[p], &sn, &cs);
+    const float c = (float)cs * mag, s = (float)sn * mag;
+    const float a = buf[2 * p], b = buf[2 * p + 1];
+    buf[2 * p] = a * c - b * s;
+    buf[2 * p + 1] = b * c + a * s;
+  }
+  __syncthreads();
+  T *dst = is_q ? q + (long)t * q_stride + (long)y * D
+                : k_cache + (slot_mapping[t] * G + (y - H)) * D;
+  for (int i = lane; i < D; i += QK_BLOCK)
+    dst[i] = ScalarOps<T>::from_f32(buf[i]);
+}
+
+// ------------------------------------------------------------------
+// grid (tokens, H); one workgroup = one (query token, query head).
+// Visible keys are enumerated as kept-first [0, n_keep) followed by the
+// window [lo, i]; tiles of ATT_BLOCK keys: one score per thread, online
+// softmax across tiles, then P.V with threads laid out as
+// (key part) x (value column).
+template <typename T, int CT>  // CT: column threads, pow2 >= min(Dv,256)
+__global__ __launch_bounds__(ATT_BLOCK) void window_attention_kernel(
+    T *__restrict__ out, const T *__restrict__ q, long q_stride,
+    const T *__restrict__ gate, long gate_stride,
+    const T *__restrict__ k_cache, const T *__restrict__ v_cache,
+    const int *__restrict__ block_table, int bt_stride,
+    const int *__restrict__ seq_lens, const int *__restrict__ qsl, int B,
+    int H, int G, int D, int Dv, int page, float scale, int window,
+    int keep_first, int sink) {
+  constexpr int PARTS = ATT_BLOCK / CT;
+  constexpr int NC = 2;  // columns per thread when Dv > CT (Dv <= 512)
+  extern __shared__ float smem[];
+  float *qs = smem;                 // [D]
+  float *ps = qs + ((D + 3) & ~3);  // [ATT_BLOCK] probabilities
+  long *rows = reinterpret_cast<long *>(ps + ATT_BLOCK);  // [ATT_BLOCK]
+  float *accs = reinterpret_cast<float *>(rows + ATT_BLOCK);  // [PARTS][NC*CT]
+  __shared__ float red[ATT_BLOCK / WAVE_SIZE];
+  __shared__ float bcast;
+
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x;
+  // which sequence owns token t: largest b with qsl[b] <= t
+  int lo_b = 0, hi_b = B - 1;
+  while (lo_b < hi_b) {
+    const int mid = (lo_b + hi_b + 1) >> 1;
+    if (qsl[mid] <= t) lo_b = mid; else hi_b = mid - 1;
+  }
+  const int b = lo_b;
+  // sequence b holds seq_lens[b] tokens after this step; its new tokens
+  // are rows qsl[b]..qsl[b+1]-1, so row t sits at position
+  const int i = seq_lens[b] - (qsl[b + 1] - t);
+  const int g = h / (H / G);
+  const int *bt = block_table + (long)b * bt_stride;
+
+  for (int d = tid; d < D; d += ATT_BLOCK)
+    qs[d] = ScalarOps<T>::to_f32(q[(long)t * q_stride + (long)h * D + d]);
+
+  const int lo = (window > 0 && i - window + 1 > 0) ? i - window + 1 : 0;
+  const int n_keep = keep_first < lo ? keep_first : lo;
+  const int total = n_keep + (i - lo + 1);
+
+  float m = sink ? 0.f : -INFINITY;
+  float l = sink ? 1.f : 0.f;
+  float acc[NC] = {0.f, 0.f};
+  const int col = tid % CT, part = tid / CT;
+  __syncthreads();
+
+  for (int base = 0; base < total; base += ATT_BLOCK) {
+    const int vi = base + tid;
+    float s = -INFINITY;
+    __syncthreads();  // the last tile's ps/rows/red are done with
+    if (vi < total) {
+      const int j = vi < n_keep ? vi : lo + (vi - n_keep);
+      const long row = (long)bt[j / page] * page + j % page;
+      rows[tid] = row;
+      const T *kr = k_cache + (row * G + g) * D;
+      float dot = 0.f;
+      for (int d = 0; d < D; ++d) dot += qs[d] * ScalarOps<T>::to_f32(kr[d]);
+      s = dot * scale;
+    }
+    // tile max -> new running max
+    float tm = wave_reduce_max(s);
+    if ((tid & 63) == 0) red[tid >> 6] = tm;
+    __syncthreads();
+    if (tid == 0) {
+      float x = red[0];
+      for (int w = 1; w < ATT_BLOCK / WAVE_SIZE; ++w) x = fmaxf(x, red[w]);
+      bcast = fmaxf(m, x);
+    }
+    __syncthreads();
+    const float m_new = bcast;
+    const float p = vi < total ? expf(s - m_new) : 0.f;
+    ps[tid] = p;
+    float psum = wave_reduce_sum(p);
+    __syncthreads();
+    if ((tid & 63) == 0) red[tid >> 6] = psum;
+    __syncthreads();
+    float tsum = 0.f;
+    for (int w = 0; w < ATT_BLOCK / WAVE_SIZE; ++w) tsum += red[w];
+    const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
+    l = l * corr + tsum;
+    m = m_new;
+    const int n_tile = total - base < ATT_BLOCK ? total - base : ATT_BLOCK;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc[c] *= corr;
+    for (int jj = part; jj < n_tile; jj += PARTS) {
+      const float pj = ps[jj];
+      const T *vr = v_cache + (rows[jj] * G + g) * Dv;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int d = col + c * CT;
+        if (d < Dv) acc[c] += pj * ScalarOps<T>::to_f32(vr[d]);
+      }
+    }
+  }
+  // reduce the key parts
+  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < NC; ++c) accs[(part * NC + c) * CT + col] = acc[c];
+  __syncthreads();
+  if (part == 0) {
+    const float inv_l = 1.0f / l;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int d = col + c * CT;
+      if (d >= Dv) continue;
+      float o = 0.f;
+      for (int pp = 0; pp < PARTS; ++pp) o += accs[(pp * NC + c) * CT + col];
+      o *= inv_l;
+      if (gate != nullptr) {
+        const float z = ScalarOps<T>::to_f32(
+            gate[(long)t * gate_stride + (long)h * Dv + d]);
+        o *= 1.0f / (1.0f + expf(-z));
+      }
+      out[((long)t * H + h) * Dv + d] = ScalarOps<T>::from_f32(o);
+    }
+  }
+}
+
+bool rows_ok(const torch::Tensor &t) {
+  return t.dim() == 2 && t.stride(1) == 1;
+}
+
+}  // namespace
+
+void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
+                        c10::optional<torch::Tensor> v, torch::Tensor q_w,
+                        c10::optional<torch::Tensor> k_w,
+                        torch::Tensor positions, torch::Tensor slot_mapping,
+                        torch::Tensor freqs, double mag, long rot_dims,
+                        c10::optional<torch::Tensor> k_cache,
+                        c10::optional<torch::Tensor> v_cache, long H, long G,
+                        long D, long Dv, double eps) {
+  const long T = q.size(0);
+  if (T == 0) return;
+  const auto st = q.scalar_type();
+  TORCH_CHECK(q.is_cuda() && rows_ok(q) && q.size(1) == H * D);
+  TORCH_CHECK(q_w.scalar_type() == st && q_w.numel() == D &&
+              q_w.is_contiguous());
+  TORCH_CHECK(positions.scalar_type() == at::kLong &&
+              positions.is_contiguous() && positions.numel() >= T);
+  TORCH_CHECK(freqs.scalar_type() == at::kDouble && freqs.is_contiguous() &&
+              freqs.numel() * 2 >= rot_dims);
+  TORCH_CHECK(rot_dims >= 0 && rot_dims <= D && rot_dims % 2 == 0,
+              "rotary dims must be even and <= head dim");
+  TORCH_CHECK(D * 4 <= 32 * 1024);
+  const bool own = k.has_value();
+  const void *kp = nullptr, *vp = nullptr, *kwp = nullptr;
+  void *kcp = nullptr, *vcp = nullptr;
+  long ks = 0, vs = 0;
+  if (own) {
+    TORCH_CHECK(v.has_value() && k_w.has_value() && k_cache.has_value() &&
+                v_cache.has_value());
+    TORCH_CHECK(rows_ok(*k) && k->size(0) == T && k->size(1) == G * D &&
+                k->scalar_type() == st);
+    TORCH_CHECK(rows_ok(*v) && v->size(0) == T && v->size(1) == G * Dv &&
+                v->scalar_type() == st);
+    TORCH_CHECK(k_w->scalar_type() == st && k_w->numel() == D);
+    TORCH_CHECK(k_cache->is_contiguous() && v_cache->is_contiguous() &&
+                k_cache->scalar_type() == st && v_cache->scalar_type() == st);
+    TORCH_CHECK(k_cache->dim() == 4 && k_cache->size(2) == G &&
+                k_cache->size(3) == D && v_cache->size(2) == G &&
+                v_cache->size(3) == Dv, "cache geometry mismatch");
+    TORCH_CHECK(slot_mapping.scalar_type() == at::kLong &&
+                slot_mapping.is_contiguous() && slot_mapping.numel() >= T);
+    kp = k->data_ptr(); vp = v->data_ptr(); kwp = k_w->data_ptr();
+    kcp = k_cache->data_ptr(); vcp = v_cache->data_ptr();
+    ks = k->stride(0); vs = v->stride(0);
+  }
+  const int gy = own ? H + 2 * G : H;
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(TT)                                                              \
+  hipLaunchKernelGGL((qk_norm_rope_store_kernel<TT>), dim3(T, gy),           \
+                     dim3(QK_BLOCK), D * sizeof(float), stream,              \
+                     (TT *)q.data_ptr(), (long)q.stride(0), (const TT *)kp,  \
+                     ks, (const TT *)vp, vs, (const TT *)q_w.data_ptr(),     \
+                     (const TT *)kwp, positions.data_ptr<long>(),            \
+                     own ? slot_mapping.data_ptr<long>() : nullptr,          \
+                     freqs.data_ptr<double>(), (float)mag, (int)rot_dims,    \
+                     (TT *)kcp, (TT *)vcp, (int)H, (int)G, (int)D, (int)Dv,  \
+                     (float)eps)
+  if (st == at::kBFloat16) RUN(__hip_bfloat16);
+  else if (st == at::kFloat) RUN(float);
+  else TORCH_CHECK(false, "qk_norm_rope_store: bf16 or fp32");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+void window_attention(torch::Tensor out, torch::Tensor q,
+                      c10::optional<torch::Tensor> gate,
+                      torch::Tensor k_cache, torch::Tensor v_cache,
+                      torch::Tensor block_table, torch::Tensor seq_lens,
+                      torch::Tensor query_start_loc, double scale,
+                      long window, long keep_first, bool sink) {
+  const long T = q.size(0);
+  if (T == 0) return;
+  const auto st = q.scalar_type();
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4);
+  const int page = k_cache.size(1), G = k_cache.size(2), D = k_cache.size(3);
+  const int Dv = v_cache.size(3);
+  TORCH_CHECK(rows_ok(q) && q.size(1) % D == 0);
+  const int H = q.size(1) / D;
+  TORCH_CHECK(H % G == 0, "query heads must be a multiple of kv heads");
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.scalar_type() == st && v_cache.scalar_type() == st);
+  TORCH_CHECK(v_cache.size(1) == page && v_cache.size(2) == G);
+  TORCH_CHECK(out.is_contiguous() && out.scalar_type() == st &&
+              out.numel() == T * H * Dv);
+  TORCH_CHECK(block_table.scalar_type() == at::kInt && block_table.dim() == 2 &&
+              block_table.stride(1) == 1);
+  TORCH_CHECK(seq_lens.scalar_type() == at::kInt && seq_lens.is_contiguous());
+  TORCH_CHECK(query_start_loc.scalar_type() == at::kInt &&
+              query_start_loc.is_contiguous());
+  const int B = seq_lens.numel();
+  TORCH_CHECK(query_start_loc.numel() >= B + 1 && block_table.size(0) >= B);
+  TORCH_CHECK(Dv <= 512, "window_attention: value size <= 512");
+  const void *gp = nullptr;
+  long gs = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(rows_ok(*gate) && gate->size(0) == T &&
+                gate->size(1) == H * Dv && gate->scalar_type() == st);
+    gp = gate->data_ptr();
+    gs = gate->stride(0);
+  }
+  int ct = 16;
+  while (ct < Dv && ct < 256) ct *= 2;
+  const int parts = ATT_BLOCK / ct;
+  const size_t lds = (((D + 3) & ~3) + ATT_BLOCK) * sizeof(float) +
+                     ATT_BLOCK * sizeof(long) +
+                     (size_t)parts * 2 * ct * sizeof(float);
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(TT, CTV)                                                         \
+  hipLaunchKernelGGL((window_attention_kernel<TT, CTV>), dim3(T, H),         \
+                     dim3(ATT_BLOCK), lds, stream, (TT *)out.data_ptr(),     \
+                     (const TT *)q.data_ptr(), (long)q.stride(0),            \
+                     (const TT *)gp, gs, (const TT *)k_cache.data_ptr(),     \
+                     (const TT *)v_cache.data_ptr(),                         \
+                     block_table.data_ptr<int>(), (int)block_table.stride(0), \
+                     seq_lens.data_ptr<int>(),                               \
+                     query_start_loc.data_ptr<int>(), B, H, G, D, Dv, page,  \
+                     (float)scale, (int)window, (int)keep_first,             \
+                     sink ? 1 : 0)
+#define RUN_CT(TT)                                                           \
+  switch (ct) {                                                              \
+    case 16: RUN(TT, 16); break;                                             \
+    case 32: RUN(TT, 32); break;                                             \
+    case 64: RUN(TT, 64); break;                                             \
+    case 128: RUN(TT, 128); break;                                           \
+    default: RUN(TT, 256); break;                                            \
+  }
+  if (st == at::kBFloat16) { RUN_CT(__hip_bfloat16) }
+  else if (st == at::kFloat) { RUN_CT(float) }
+  else TORCH_CHECK(false, "window_attention: bf16 or fp32");
+#undef RUN_CT
+#undef RUN
+  HIP_CHECK_KERNEL();
+}

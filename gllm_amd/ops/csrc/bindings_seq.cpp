@@ -1,0 +1,68 @@
+// Python bindings for the dtype-generic sequence-mixer kernels
+// (gllm_amd._kernels_seq): fp32-residual layer norm, windowed sink
+// attention, varlen gated delta rule, plus the grouped MoE GEMM and the
+// gated activations they are served with.
+#include <torch/extension.h>
+
+void layernorm_f32(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                   torch::Tensor b, double eps);
+void residual_layernorm(torch::Tensor x, torch::Tensor y,
+                        torch::Tensor w_post, torch::Tensor b_post,
+                        c10::optional<torch::Tensor> h,
+                        c10::optional<torch::Tensor> w_pre,
+                        c10::optional<torch::Tensor> b_pre, double eps);
+void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
+                        c10::optional<torch::Tensor> v, torch::Tensor q_w,
+                        c10::optional<torch::Tensor> k_w,
+                        torch::Tensor positions, torch::Tensor slot_mapping,
+                        torch::Tensor freqs, double mag, long rot_dims,
+                        c10::optional<torch::Tensor> k_cache,
+                        c10::optional<torch::Tensor> v_cache, long H, long G,
+                        long D, long Dv, double eps);
+void window_attention(torch::Tensor out, torch::Tensor q,
+                      c10::optional<torch::Tensor> gate,
+                      torch::Tensor k_cache, torch::Tensor v_cache,
+                      torch::Tensor block_table, torch::Tensor seq_lens,
+                      torch::Tensor query_start_loc, double scale,
+                      long window, long keep_first, bool sink);
+void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                      torch::Tensor conv_state, torch::Tensor slots,
+                      torch::Tensor has_init, torch::Tensor query_start_loc);
+void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
+                       torch::Tensor v, torch::Tensor a, torch::Tensor b,
+                       torch::Tensor A_log, torch::Tensor dt_bias,
+                       torch::Tensor state, torch::Tensor slots,
+                       torch::Tensor has_init, torch::Tensor query_start_loc,
+                       double q_scale);
+void rms_gate(torch::Tensor out, torch::Tensor o, torch::Tensor z,
+              torch::Tensor w, long H, double eps);
+// shared with the full extension (moe.hip, elementwise.hip)
+void silu_and_mul(torch::Tensor out, torch::Tensor x);
+void moe_align(torch::Tensor topk_ids, long E_local, long expert_start,
+               long block_m, torch::Tensor sorted_ids,
+               torch::Tensor expert_blocks, torch::Tensor n_post_pad);
+void moe_gemm(torch::Tensor C, torch::Tensor A, torch::Tensor W,
+              torch::Tensor sorted_ids, torch::Tensor expert_blocks,
+              torch::Tensor n_post_pad,
+              c10::optional<torch::Tensor> topk_weights, long n_pairs,
+              long topk, long block_m, bool scatter);
+void moe_sum(torch::Tensor out, torch::Tensor pair_out, long topk);
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("layernorm_f32", &layernorm_f32, "h = LN(x fp32) in the model dtype");
+  m.def("residual_layernorm", &residual_layernorm,
+        "x += LN_post(y); optionally h = LN_pre(x)");
+  m.def("qk_norm_rope_store", &qk_norm_rope_store,
+        "per-head q/k RMS norm + interleaved rotary + paged K/V store");
+  m.def("window_attention", &window_attention,
+        "ragged paged attention: window + kept first tokens + sink + gate");
+  m.def("causal_conv_silu", &causal_conv_silu,
+        "ragged short causal conv + silu with per-slot state");
+  m.def("delta_rule_varlen", &delta_rule_varlen,
+        "ragged gated delta rule, fp32 state in registers");
+  m.def("rms_gate", &rms_gate, "o / rms(o) * w * silu(z) per head");
+  m.def("silu_and_mul", &silu_and_mul, "silu(x[:d]) * x[d:]");
+  m.def("moe_align", &moe_align, "device-side moe_align_block_size");
+  m.def("moe_gemm", &moe_gemm, "grouped MFMA GEMM over sorted pairs");
+  m.def("moe_sum", &moe_sum, "sum pair outputs over topk");
+}

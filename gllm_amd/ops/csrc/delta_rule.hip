@@ -1,0 +1,339 @@
+// Gated delta rule over ragged batches, any head geometry, gfx950.
+//
+// Dtype-generic (projections T = bf16 or fp32; unit norms, gates, decay
+// and the recurrent state are fp32 always). One code path serves prompt
+// portions of any length and single decode tokens in the same launch,
+// so a position's result never depends on how its sequence was cut.
+//
+//   causal_conv_silu   short causal depthwise convolution over time with
+//                      silu; the taps-1 inputs before a portion come from
+//                      the per-slot conv state
+//   conv_state_update  rolls the conv state to the portion's last inputs
+//   delta_rule_varlen  per (sequence, value head): for each token
+//                        S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;
+//                        o = S^T q
+//                      with q, k unit-normalised per head (q also scaled),
+//                      beta = sigmoid(b), g = exp(-exp(A_log) softplus(a + dt)).
+//                      A wavefront owns 16 state columns; its 64 lanes are
+//                      4 key-slices x 16 columns, reductions over the key
+//                      axis are two lane shuffles, and waves never meet at a
+//                      barrier: the state column block lives in registers
+//                      for the whole portion.
+//   rms_gate           o / rms(o) * w * silu(z) per head
+//
+// State layouts: conv [slots, C, taps-1] (oldest first), recurrent
+// [slots, H, Dk, Dv] fp32.
+
+#include <torch/extension.h>
+#include <ATen/cuda/CUDAContext.h>
+#include "common.h"
+
+namespace {
+
+constexpr int MAX_TAPS = 8;
+
+DEV_INLINE int find_seq(const int *__restrict__ qsl, int B, int t) {
+  int lo = 0, hi = B - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (qsl[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+DEV_INLINE float silu_f(float z) { return z / (1.0f + expf(-z)); }
+
+// grid (tokens, ceil(C / 256))
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_silu_kernel(
+    T *__restrict__ out, const T *__restrict__ x, long x_stride,
+    const T *__restrict__ w, const T *__restrict__ state,
+    const long *__restrict__ slots, const int *__restrict__ has_init,
+    const int *__restrict__ qsl, int B, int C, int taps) {
+  const int t = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int b = find_seq(qsl, B, t);
+  const int r = t - qsl[b];  // offset inside this portion
+  const bool init = has_init[b] != 0;
+  const T *st = state + ((long)slots[b] * C + c) * (taps - 1);
+  float acc = 0.f;
+  for (int tap = 0; tap < taps; ++tap) {
+    const int rel = r - (taps - 1 - tap);
+    float xv;
+    if (rel >= 0)
+      xv = ScalarOps<T>::to_f32(x[(long)(qsl[b] + rel) * x_stride + c]);
+    else
+      xv = init ? ScalarOps<T>::to_f32(st[taps - 1 + rel]) : 0.f;
+    acc += xv * ScalarOps<T>::to_f32(w[(long)c * taps + tap]);
+  }
+  // the activation output feeds 16-bit consumers in bf16 serving
+  out[(long)t * C + c] = ScalarOps<T>::from_f32(silu_f(acc));
+}
+
+// grid (B, ceil(C / 256)); each thread owns one (sequence, channel) state
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(
+    T *__restrict__ state, const T *__restrict__ x, long x_stride,
+    const long *__restrict__ slots, const int *__restrict__ has_init,
+    const int *__restrict__ qsl, int C, int taps) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int start = qsl[b], n = qsl[b + 1] - qsl[b];
+  const bool init = has_init[b] != 0;
+  T *st = state + ((long)slots[b] * C + c) * (taps - 1);
+  T next[MAX_TAPS];
+  for (int i = 0; i < taps - 1; ++i) {
+    const int rel = n - (taps - 1) + i;
+    if (rel >= 0) next[i] = x[(long)(start + rel) * x_stride + c];
+    else next[i] = init ? st[taps - 1 + rel] : ScalarOps<T>::from_f32(0.f);
+  }
+  for (int i = 0; i < taps - 1; ++i) st[i] = next[i];
+}
+
+// grid (B, H, ceil(Dv / 64)), block 256 = 4 independent waves.
+// KP = key elements per lane = ceil(Dk / 4); lane (part, col) holds
+// S[part + 4 r][col] for r < KP.
+template <typename T, int KP>
+__global__ __launch_bounds__(256) void delta_rule_varlen_kernel(
+    float *__restrict__ o, const T *__restrict__ q, const T *__restrict__ k,
+    const T *__restrict__ v, long qkv_stride, const T *__restrict__ a,
+    const T *__restrict__ bproj, long ab_stride,
+    const float *__restrict__ A_log, const float *__restrict__ dt_bias,
+    float *__restrict__ state, const long *__restrict__ slots,
+    const int *__restrict__ has_init, const int *__restrict__ qsl, int H,
+    int G, int Dk, int Dv, float q_scale) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = blockIdx.z * 64 + wave * 16 + (lane & 15);
+  const int part = lane >> 4;
+  const int g = h / (H / G);
+  const int start = qsl[b], end = qsl[b + 1];
+  const bool live = col < Dv;
+  const int colc = live ? col : Dv - 1;  // clamp loads, mask stores
+  if (blockIdx.z * 64 + wave * 16 >= Dv) return;  // whole wave idle
+
+  float *sp = state + ((long)slots[b] * H + h) * Dk * Dv;
+  float S[KP];
+  const bool init = has_init[b] != 0;
+#pragma unroll
+  for (int r = 0; r < KP; ++r) {
+    const int i = part + 4 * r;
+    S[r] = (init && i < Dk) ? sp[(long)i * Dv + colc] : 0.f;
+  }
+  const float neg_rate = -expf(A_log[h]);
+  const float dtb = dt_bias[h];
+
+  for (int t = start; t < end; ++t) {
+    const T *qr = q + (long)t * qkv_stride + (long)g * Dk;
+    const T *kr = k + (long)t * qkv_stride + (long)g * Dk;
+    float kn[KP], qn[KP];
+    float sk = 0.f, sq = 0.f;
+#pragma unroll
+    for (int r = 0; r < KP; ++r) {
+      const int i = part + 4 * r;
+      const float kv = i < Dk ? ScalarOps<T>::to_f32(kr[i]) : 0.f;
+      const float qv = i < Dk ? ScalarOps<T>::to_f32(qr[i]) : 0.f;
+      kn[r] = kv;
+      qn[r] = qv;
+      sk += kv * kv;
+      sq += qv * qv;
+    }
+    sk += __shfl_xor(sk, 16, 64);
+    sk += __shfl_xor(sk, 32, 64);
+    sq += __shfl_xor(sq, 16, 64);
+    sq += __shfl_xor(sq, 32, 64);
+    const float ik = 1.0f / sqrtf(sk + 1e-6f);
+    const float iq = q_scale / sqrtf(sq + 1e-6f);
+    const float vv =
+        ScalarOps<T>::to_f32(v[(long)t * qkv_stride + (long)h * Dv + colc]);
+    const float av = ScalarOps<T>::to_f32(a[(long)t * ab_stride + h]) + dtb;
+    const float bv = ScalarOps<T>::to_f32(bproj[(long)t * ab_stride + h]);
+    // softplus without overflow: max(x, 0) + log1p(exp(-|x|))
+    const float sp_a = fmaxf(av, 0.f) + log1pf(expf(-fabsf(av)));
+    const float gdec = expf(neg_rate * sp_a);
+    const float beta = 1.0f / (1.0f + expf(-bv));
+    float sk_dot = 0.f;
+#pragma unroll
+    for (int r = 0; r < KP; ++r) {
+      kn[r] *= ik;
+      qn[r] *= iq;
+      S[r] *= gdec;
+      sk_dot += S[r] * kn[r];
+    }
+    sk_dot += __shfl_xor(sk_dot, 16, 64);
+    sk_dot += __shfl_xor(sk_dot, 32, 64);
+    const float u = beta * (vv - sk_dot);
+    float od = 0.f;
+#pragma unroll
+    for (int r = 0; r < KP; ++r) {
+      S[r] += kn[r] * u;
+      od += S[r] * qn[r];
+    }
+    od += __shfl_xor(od, 16, 64);
+    od += __shfl_xor(od, 32, 64);
+    if (live && part == 0) o[((long)t * H + h) * Dv + col] = od;
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < KP; ++r) {
+      const int i = part + 4 * r;
+      if (i < Dk) sp[(long)i * Dv + col] = S[r];
+    }
+  }
+}
+
+// grid (tokens * H); block 64: out = o / rms(o) * w * silu(z)
+template <typename T>
+__global__ __launch_bounds__(64) void rms_gate_kernel(
+    T *__restrict__ out, const float *__restrict__ o,
+    const T *__restrict__ z, long z_stride, const T *__restrict__ w,
+    int H, int Dv, float eps) {
+  const long th = blockIdx.x;
+  const long t = th / H;
+  const int h = th % H;
+  const float *orow = o + th * Dv;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < Dv; d += 64) ss += orow[d] * orow[d];
+  ss = wave_reduce_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / Dv + eps);
+  for (int d = threadIdx.x; d < Dv; d += 64) {
+    const float zz = ScalarOps<T>::to_f32(z[t * z_stride + (long)h * Dv + d]);
+    out[th * Dv + d] = ScalarOps<T>::from_f32(
+        orow[d] * inv * ScalarOps<T>::to_f32(w[d]) * silu_f(zz));
+  }
+}
+
+bool rows_ok(const torch::Tensor &t) {
+  return t.dim() == 2 && t.stride(1) == 1;
+}
+
+}  // namespace
+
+void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                      torch::Tensor conv_state, torch::Tensor slots,
+                      torch::Tensor has_init, torch::Tensor query_start_loc) {
+  const long T = x.size(0);
+  const int C = x.size(1);
+  const int taps = w.size(1);
+  const int B = slots.numel();
+  if (T == 0) return;
+  const auto st = x.scalar_type();
+  TORCH_CHECK(rows_ok(x) && out.is_contiguous() && out.scalar_type() == st &&
+              out.numel() == T * C);
+  TORCH_CHECK(w.is_contiguous() && w.size(0) == C && w.scalar_type() == st);
+  TORCH_CHECK(taps >= 1 && taps <= MAX_TAPS, "conv taps must be 1..8");
+  TORCH_CHECK(conv_state.is_contiguous() && conv_state.scalar_type() == st &&
+              conv_state.dim() == 3 && conv_state.size(1) == C &&
+              conv_state.size(2) == std::max(taps - 1, 1));
+  TORCH_CHECK(slots.scalar_type() == at::kLong && slots.is_contiguous());
+  TORCH_CHECK(has_init.scalar_type() == at::kInt && has_init.numel() == B);
+  TORCH_CHECK(query_start_loc.scalar_type() == at::kInt &&
+              query_start_loc.numel() >= B + 1);
+  auto stream = at::cuda::getCurrentCUDAStream();
+  const int cy = (C + 255) / 256;
+#define RUN(TT)                                                              \
+  hipLaunchKernelGGL((causal_conv_silu_kernel<TT>), dim3(T, cy), dim3(256),  \
+                     0, stream, (TT *)out.data_ptr(),                        \
+                     (const TT *)x.data_ptr(), (long)x.stride(0),            \
+                     (const TT *)w.data_ptr(),                               \
+                     (const TT *)conv_state.data_ptr(),                      \
+                     slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
+                     query_start_loc.data_ptr<int>(), B, C, taps);           \
+  if (taps > 1)                                                              \
+    hipLaunchKernelGGL((conv_state_update_kernel<TT>), dim3(B, cy),          \
+                       dim3(256), 0, stream, (TT *)conv_state.data_ptr(),    \
+                       (const TT *)x.data_ptr(), (long)x.stride(0),          \
+                       slots.data_ptr<long>(), has_init.data_ptr<int>(),     \
+                       query_start_loc.data_ptr<int>(), C, taps)
+  if (st == at::kBFloat16) { RUN(__hip_bfloat16); }
+  else if (st == at::kFloat) { RUN(float); }
+  else TORCH_CHECK(false, "causal_conv_silu: bf16 or fp32");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
+                       torch::Tensor v, torch::Tensor a, torch::Tensor b,
+                       torch::Tensor A_log, torch::Tensor dt_bias,
+                       torch::Tensor state, torch::Tensor slots,
+                       torch::Tensor has_init, torch::Tensor query_start_loc,
+                       double q_scale) {
+  const long T = q.size(0);
+  if (T == 0) return;
+  const auto st = q.scalar_type();
+  TORCH_CHECK(state.dim() == 4 && state.scalar_type() == at::kFloat &&
+              state.is_contiguous());
+  const int H = state.size(1), Dk = state.size(2), Dv = state.size(3);
+  TORCH_CHECK(rows_ok(q) && rows_ok(k) && rows_ok(v) && rows_ok(a) &&
+              rows_ok(b));
+  TORCH_CHECK(k.scalar_type() == st && v.scalar_type() == st &&
+              a.scalar_type() == st && b.scalar_type() == st);
+  TORCH_CHECK(q.size(1) % Dk == 0 && k.size(1) == q.size(1));
+  const int G = q.size(1) / Dk;
+  TORCH_CHECK(G > 0 && H % G == 0 && v.size(1) == (long)H * Dv);
+  TORCH_CHECK(q.stride(0) == k.stride(0) && q.stride(0) == v.stride(0),
+              "q, k, v must share a row stride (slices of one buffer)");
+  TORCH_CHECK(a.size(1) == H && b.size(1) == H && a.stride(0) == b.stride(0));
+  TORCH_CHECK(k.size(0) == T && v.size(0) == T && a.size(0) == T &&
+              b.size(0) == T);
+  TORCH_CHECK(A_log.scalar_type() == at::kFloat && A_log.numel() == H &&
+              dt_bias.scalar_type() == at::kFloat && dt_bias.numel() == H);
+  TORCH_CHECK(o.scalar_type() == at::kFloat && o.is_contiguous() &&
+              o.numel() == T * H * Dv);
+  const int B = slots.numel();
+  TORCH_CHECK(slots.scalar_type() == at::kLong && slots.is_contiguous());
+  TORCH_CHECK(has_init.scalar_type() == at::kInt && has_init.numel() == B);
+  TORCH_CHECK(query_start_loc.scalar_type() == at::kInt &&
+              query_start_loc.numel() >= B + 1);
+  TORCH_CHECK(Dk <= 256, "delta rule: key size <= 256");
+  auto stream = at::cuda::getCurrentCUDAStream();
+  const dim3 grid(B, H, (Dv + 63) / 64);
+#define RUN(TT, KPV)                                                         \
+  hipLaunchKernelGGL((delta_rule_varlen_kernel<TT, KPV>), grid, dim3(256),   \
+                     0, stream, o.data_ptr<float>(),                         \
+                     (const TT *)q.data_ptr(), (const TT *)k.data_ptr(),     \
+                     (const TT *)v.data_ptr(), (long)q.stride(0),            \
+                     (const TT *)a.data_ptr(), (const TT *)b.data_ptr(),     \
+                     (long)a.stride(0), A_log.data_ptr<float>(),             \
+                     dt_bias.data_ptr<float>(), state.data_ptr<float>(),     \
+                     slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
+                     query_start_loc.data_ptr<int>(), H, G, Dk, Dv,          \
+                     (float)q_scale)
+#define RUN_KP(TT)                                                           \
+  if (Dk <= 32) RUN(TT, 8);                                                  \
+  else if (Dk <= 64) RUN(TT, 16);                                            \
+  else if (Dk <= 128) RUN(TT, 32);                                           \
+  else RUN(TT, 64)
+  if (st == at::kBFloat16) { RUN_KP(__hip_bfloat16); }
+  else if (st == at::kFloat) { RUN_KP(float); }
+  else TORCH_CHECK(false, "delta_rule_varlen: bf16 or fp32");
+#undef RUN_KP
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+void rms_gate(torch::Tensor out, torch::Tensor o, torch::Tensor z,
+              torch::Tensor w, long H, double eps) {
+  const int Dv = w.numel();
+  const long rows = o.numel() / std::max(Dv, 1);
+  if (rows == 0) return;
+  const auto st = out.scalar_type();
+  TORCH_CHECK(o.scalar_type() == at::kFloat && o.is_contiguous());
+  TORCH_CHECK(out.is_contiguous() && out.numel() == o.numel());
+  TORCH_CHECK(rows_ok(z) && z.scalar_type() == st && z.size(1) == H * Dv &&
+              z.size(0) * H == rows);
+  TORCH_CHECK(w.scalar_type() == st && w.is_contiguous());
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(TT)                                                              \
+  hipLaunchKernelGGL((rms_gate_kernel<TT>), dim3(rows), dim3(64), 0, stream, \
+                     (TT *)out.data_ptr(), o.data_ptr<float>(),              \
+                     (const TT *)z.data_ptr(), (long)z.stride(0),            \
+                     (const TT *)w.data_ptr(), (int)H, Dv, (float)eps)
+  if (st == at::kBFloat16) RUN(__hip_bfloat16);
+  else if (st == at::kFloat) RUN(float);
+  else TORCH_CHECK(false, "rms_gate: bf16 or fp32");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}

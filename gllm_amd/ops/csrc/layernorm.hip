@@ -1,0 +1,159 @@
+// LayerNorm (weight + bias) over an fp32 residual stream, gfx950.
+//
+// The residual stream of a sandwich-norm decoder (norm before AND after
+// every sublayer) is kept in fp32 while the sublayers run in the model
+// dtype T (bf16 or fp32). Two kernels cover a whole layer boundary:
+//
+//   layernorm_f32:      h = LN_pre(x)                       x fp32 -> h T
+//   residual_layernorm: x += LN_post(y); h = LN_pre(x)      y T, x fp32
+//
+// One workgroup per token row; the row lives in LDS as fp32 between the
+// mean, variance (mean of squared deviations, two passes: no E[x^2] -
+// E[x]^2 cancellation) and normalize passes, so HBM sees each operand
+// once. Statistics and the residual sum are fp32 whatever T is.
+
+#include <torch/extension.h>
+#include <ATen/cuda/CUDAContext.h>
+#include "common.h"
+
+namespace {
+
+constexpr int LN_BLOCK = 256;
+
+DEV_INLINE float ln_block_sum(float v, float *red) {
+  __syncthreads();  // red may still be read from a previous reduction
+  return block_reduce_sum<LN_BLOCK>(v, red);
+}
+
+// normalize the LDS row in place: row = (row - mean) / sqrt(var + eps) * w + b
+template <typename T>
+DEV_INLINE void ln_row(float *row, const T *__restrict__ w,
+                       const T *__restrict__ b, float eps, int width,
+                       float *red) {
+  float s = 0.f;
+  for (int i = threadIdx.x; i < width; i += LN_BLOCK) s += row[i];
+  const float mean = ln_block_sum(s, red) / width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += LN_BLOCK) {
+    const float d = row[i] - mean;
+    ss += d * d;
+  }
+  const float var = ln_block_sum(ss, red) / width;
+  const float inv = 1.0f / sqrtf(var + eps);
+  for (int i = threadIdx.x; i < width; i += LN_BLOCK)
+    row[i] = (row[i] - mean) * inv * ScalarOps<T>::to_f32(w[i]) +
+             ScalarOps<T>::to_f32(b[i]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(LN_BLOCK) void layernorm_f32_kernel(
+    T *__restrict__ out, const float *__restrict__ x,
+    const T *__restrict__ w, const T *__restrict__ b, float eps, int width) {
+  extern __shared__ float row[];
+  __shared__ float red[LN_BLOCK / WAVE_SIZE];
+  const long base = (long)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += LN_BLOCK) row[i] = x[base + i];
+  __syncthreads();
+  ln_row<T>(row, w, b, eps, width, red);
+  for (int i = threadIdx.x; i < width; i += LN_BLOCK)
+    out[base + i] = ScalarOps<T>::from_f32(row[i]);
+}
+
+// x += LN(y; w_post, b_post); optionally h = LN(x; w_pre, b_pre)
+template <typename T>
+__global__ __launch_bounds__(LN_BLOCK) void residual_layernorm_kernel(
+    float *__restrict__ x, const T *__restrict__ y, long y_stride,
+    const T *__restrict__ w_post, const T *__restrict__ b_post,
+    T *__restrict__ h, const T *__restrict__ w_pre,
+    const T *__restrict__ b_pre, float eps, int width) {
+  extern __shared__ float row[];
+  __shared__ float red[LN_BLOCK / WAVE_SIZE];
+  const long base = (long)blockIdx.x * width;
+  const T *yr = y + (long)blockIdx.x * y_stride;
+  for (int i = threadIdx.x; i < width; i += LN_BLOCK)
+    row[i] = ScalarOps<T>::to_f32(yr[i]);
+  __syncthreads();
+  ln_row<T>(row, w_post, b_post, eps, width, red);
+  for (int i = threadIdx.x; i < width; i += LN_BLOCK) {
+    const float r = x[base + i] + row[i];
+    x[base + i] = r;
+    row[i] = r;
+  }
+  if (h == nullptr) return;
+  __syncthreads();
+  ln_row<T>(row, w_pre, b_pre, eps, width, red);
+  for (int i = threadIdx.x; i < width; i += LN_BLOCK)
+    h[base + i] = ScalarOps<T>::from_f32(row[i]);
+}
+
+void check_vec(const torch::Tensor &t, int width, at::ScalarType st) {
+  TORCH_CHECK(t.is_cuda() && t.is_contiguous() && t.numel() == width &&
+              t.scalar_type() == st, "layernorm: bad weight/bias");
+}
+
+}  // namespace
+
+void layernorm_f32(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                   torch::Tensor b, double eps) {
+  TORCH_CHECK(x.scalar_type() == at::kFloat && x.is_contiguous());
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes());
+  const int width = x.size(-1);
+  const long rows = x.numel() / std::max(width, 1);
+  if (rows == 0) return;
+  TORCH_CHECK(width > 0 && width * 4 <= 64 * 1024);
+  check_vec(w, width, out.scalar_type());
+  check_vec(b, width, out.scalar_type());
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(T)                                                             \
+  hipLaunchKernelGGL((layernorm_f32_kernel<T>), dim3(rows), dim3(LN_BLOCK), \
+                     width * sizeof(float), stream, (T *)out.data_ptr(),   \
+                     x.data_ptr<float>(), (const T *)w.data_ptr(),         \
+                     (const T *)b.data_ptr(), (float)eps, width)
+  if (out.scalar_type() == at::kBFloat16) RUN(__hip_bfloat16);
+  else if (out.scalar_type() == at::kFloat) RUN(float);
+  else TORCH_CHECK(false, "layernorm_f32: bf16 or fp32 output");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+void residual_layernorm(torch::Tensor x, torch::Tensor y,
+                        torch::Tensor w_post, torch::Tensor b_post,
+                        c10::optional<torch::Tensor> h,
+                        c10::optional<torch::Tensor> w_pre,
+                        c10::optional<torch::Tensor> b_pre, double eps) {
+  TORCH_CHECK(x.scalar_type() == at::kFloat && x.is_contiguous());
+  const int width = x.size(-1);
+  const long rows = x.numel() / std::max(width, 1);
+  if (rows == 0) return;
+  TORCH_CHECK(width > 0 && width * 4 <= 64 * 1024);
+  TORCH_CHECK(y.dim() == 2 && y.size(0) == rows && y.size(1) == width &&
+              y.stride(1) == 1, "residual_layernorm: y must be [rows, width]");
+  const auto st = y.scalar_type();
+  check_vec(w_post, width, st);
+  check_vec(b_post, width, st);
+  void *hp = nullptr;
+  const void *wp = nullptr, *bp = nullptr;
+  if (h.has_value()) {
+    TORCH_CHECK(w_pre.has_value() && b_pre.has_value());
+    TORCH_CHECK(h->is_contiguous() && h->numel() == x.numel() &&
+                h->scalar_type() == st);
+    check_vec(*w_pre, width, st);
+    check_vec(*b_pre, width, st);
+    hp = h->data_ptr();
+    wp = w_pre->data_ptr();
+    bp = b_pre->data_ptr();
+  }
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(T)                                                              \
+  hipLaunchKernelGGL((residual_layernorm_kernel<T>), dim3(rows),            \
+                     dim3(LN_BLOCK), width * sizeof(float), stream,         \
+                     x.data_ptr<float>(), (const T *)y.data_ptr(),          \
+                     (long)y.stride(0), (const T *)w_post.data_ptr(),       \
+                     (const T *)b_post.data_ptr(), (T *)hp, (const T *)wp,  \
+                     (const T *)bp, (float)eps, width)
+  if (st == at::kBFloat16) RUN(__hip_bfloat16);
+  else if (st == at::kFloat) RUN(float);
+  else TORCH_CHECK(false, "residual_layernorm: bf16 or fp32 sublayer output");
+#undef RUN
+  HIP_CHECK_KERNEL();
+}

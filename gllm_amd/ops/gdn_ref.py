@@ -220,3 +220,72 @@ def rmsnorm_gated(x: torch.Tensor, z: torch.Tensor, weight: torch.Tensor,
     var = xf.pow(2).mean(-1, keepdim=True)
     n = xf * torch.rsqrt(var + eps) * weight.float()
     return (n * F.silu(z.float())).to(x.dtype)
+
+
+# ------------------------------------------------------------------
+# ragged (varlen) forms over per-slot state pools: the CPU path and the
+# kernel oracle of ops.causal_conv_silu / delta_rule_varlen / rms_gate
+def causal_conv_silu(x, w, conv_state, slots, has_init, query_start_loc):
+    """Short causal depthwise conv + silu over a ragged batch. ``x``
+    [T, C], ``w`` [C, taps] (last tap = current token), ``conv_state``
+    [slots, C, taps-1] holds each sequence's previous inputs and is
+    rolled forward in place."""
+    taps = w.shape[1]
+    qsl = query_start_loc.tolist()
+    out = torch.empty(x.shape, dtype=x.dtype)
+    for b, slot in enumerate(slots.tolist()):
+        s, e = qsl[b], qsl[b + 1]
+        if taps > 1 and bool(has_init[b]):
+            hist = conv_state[slot].t().to(x.dtype)
+        else:
+            hist = x.new_zeros(taps - 1, x.shape[1])
+        seq = torch.cat([hist, x[s:e]])
+        acc = torch.zeros(e - s, x.shape[1], dtype=torch.float32)
+        for tap in range(taps):
+            acc += seq[tap:tap + e - s].float() * w[:, tap].float()
+        out[s:e] = F.silu(acc).to(x.dtype)
+        if taps > 1:
+            conv_state[slot] = seq[seq.shape[0] - (taps - 1):].t()
+    return out
+
+
+def delta_rule_varlen(q, k, v, a, b, A_log, dt_bias, state, slots,
+                      has_init, query_start_loc, q_scale):
+    """Token-by-token gated delta rule over a ragged batch; fp32 state
+    [slots, H, Dk, Dv] updated in place. q, k [T, G*Dk] and v [T, H*Dv]
+    arrive un-normalised; unit norms, beta = sigmoid(b) and the decay
+    exp(-exp(A_log) * softplus(a + dt_bias)) are taken here in fp32."""
+    H, Dk, Dv = state.shape[1:]
+    T = q.shape[0]
+    G = q.shape[1] // Dk
+    qf = q.float().reshape(T, G, Dk)
+    kf = k.float().reshape(T, G, Dk)
+    qf = qf / torch.sqrt((qf * qf).sum(-1, keepdim=True) + 1e-6) * q_scale
+    kf = kf / torch.sqrt((kf * kf).sum(-1, keepdim=True) + 1e-6)
+    qf = qf.repeat_interleave(H // G, dim=1)
+    kf = kf.repeat_interleave(H // G, dim=1)
+    vf = v.float().reshape(T, H, Dv)
+    beta = torch.sigmoid(b.float())
+    decay = torch.exp(-torch.exp(A_log.float())
+                      * F.softplus(a.float() + dt_bias.float()))
+    out = torch.empty(T, H, Dv, dtype=torch.float32)
+    qsl = query_start_loc.tolist()
+    for i, slot in enumerate(slots.tolist()):
+        S = state[slot].clone() if bool(has_init[i]) \
+            else torch.zeros(H, Dk, Dv)
+        for t in range(qsl[i], qsl[i + 1]):
+            S = S * decay[t, :, None, None]
+            u = beta[t, :, None] * (vf[t] - torch.einsum(
+                "hkv,hk->hv", S, kf[t]))
+            S = S + kf[t, :, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hkv,hk->hv", S, qf[t])
+        state[slot] = S
+    return out
+
+
+def rms_gate(o, z, w, H, eps, dtype):
+    """Per head: o / rms(o) * w * silu(z); o fp32 [T, H, Dv]."""
+    T = o.shape[0]
+    of = o.float().reshape(T, H, -1)
+    of = of * torch.rsqrt((of * of).mean(-1, keepdim=True) + eps) * w.float()
+    return (of.reshape(T, -1) * F.silu(z.float())).to(dtype)

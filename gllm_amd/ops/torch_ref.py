@@ -254,3 +254,107 @@ def apply_repetition_penalty(logits: torch.Tensor, token_ids_per_row,
         vals = row[toks]
         row[toks] = torch.where(vals > 0, vals / p, vals * p)
     return logits
+
+
+# ------------------------------------------------------------------
+# fp32-residual layer norm / windowed sink attention (CPU path + kernel
+# oracle for ops.layernorm_f32, residual_layernorm, qk_norm_rope_store,
+# window_attention)
+def layernorm_f32(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor,
+                  eps: float, dtype) -> torch.Tensor:
+    """LayerNorm of an fp32 row with weight and bias, output in ``dtype``."""
+    xf = x.float()
+    mu = xf.mean(-1, keepdim=True)
+    d = xf - mu
+    var = (d * d).mean(-1, keepdim=True)
+    return (d * torch.rsqrt(var + eps) * w.float() + b.float()).to(dtype)
+
+
+def residual_layernorm(x: torch.Tensor, y: torch.Tensor, w_post, b_post,
+                       eps: float, pre=None):
+    """x (fp32, in place) += LN(y); returns LN_pre(x) when ``pre`` is a
+    (weight, bias) pair."""
+    x.add_(layernorm_f32(y, w_post, b_post, eps, torch.float32))
+    if pre is None:
+        return None
+    return layernorm_f32(x, pre[0], pre[1], eps, y.dtype)
+
+
+def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
+                       mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps):
+    """Per-head RMS norm (plain weight) + interleaved-pair rotary on q
+    (in place) and k; k, v land in the paged cache rows ``slot_mapping``.
+    ``k`` None: a layer that reads another layer's cache."""
+    T = q.shape[0]
+    ang = positions[:T].double()[:, None] * freqs.double()[None, :rot_dims // 2]
+    cos = (torch.cos(ang).float() * mag)[:, None, :]
+    sin = (torch.sin(ang).float() * mag)[:, None, :]
+
+    def prep(x, w, heads):
+        xf = x.float().reshape(T, heads, D)
+        xf = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps) \
+            * w.float()
+        a, b = xf[..., 0:rot_dims:2], xf[..., 1:rot_dims:2]
+        rot = torch.stack([a * cos - b * sin, b * cos + a * sin], dim=-1)
+        return torch.cat([rot.flatten(-2), xf[..., rot_dims:]], dim=-1)
+
+    q.copy_(prep(q, q_w, H).reshape(T, H * D).to(q.dtype))
+    if k is None:
+        return
+    page = k_cache.shape[1]
+    rows = slot_mapping[:T]
+    kc = k_cache.view(-1, G, D)
+    vc = v_cache.view(-1, G, Dv)
+    kc[rows] = prep(k, k_w, G).to(k_cache.dtype)
+    vc[rows] = v.reshape(T, G, Dv).to(v_cache.dtype)
+    del page
+
+
+def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
+                     query_start_loc, scale, window, keep_first, sink):
+    """Ragged paged attention: position i sees j <= i with i - j < window
+    (window <= 0: all) or j < keep_first; ``sink`` adds 1 to the softmax
+    denominator; ``gate`` multiplies the heads by sigmoid(gate)."""
+    page, G, D = k_cache.shape[1:]
+    Dv = v_cache.shape[3]
+    T = q.shape[0]
+    H = q.shape[1] // D
+    out = torch.zeros(T, H, Dv, dtype=torch.float32)
+    qsl = query_start_loc.tolist()
+    lens = seq_lens.tolist()
+    qf = q.float().reshape(T, H, D)
+    for b in range(len(lens)):
+        s, e, L = qsl[b], qsl[b + 1], lens[b]
+        if e == s:
+            continue
+        pages = block_table[b, :-(-L // page)].long()
+        kk = k_cache[pages].reshape(-1, G, D)[:L].float()
+        vv = v_cache[pages].reshape(-1, G, Dv)[:L].float()
+        pos_i = torch.arange(L - (e - s), L)[:, None]
+        pos_j = torch.arange(L)[None, :]
+        see = pos_j <= pos_i
+        if window > 0:
+            see = see & ((pos_i - pos_j < window) | (pos_j < keep_first))
+        kk = kk.repeat_interleave(H // G, dim=1)
+        vv = vv.repeat_interleave(H // G, dim=1)
+        sc = torch.einsum("ihd,jhd->hij", qf[s:e], kk) * scale
+        sc = sc.masked_fill(~see[None], float("-inf"))
+        m = sc.amax(-1, keepdim=True)
+        if sink:
+            m = m.clamp_min(0.0)
+        p = torch.exp(sc - m)
+        den = p.sum(-1, keepdim=True)
+        if sink:
+            den = den + torch.exp(-m)
+        out[s:e] = torch.einsum("hij,jhd->ihd", p / den, vv)
+    out = out.reshape(T, H * Dv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())
+    return out.to(q.dtype)
+
+
+def topk_then_softmax(logits: torch.Tensor, topk: int):
+    """MoE routing that picks the ``topk`` largest LOGITS and softmaxes
+    over the chosen ones only. Returns (weights fp32 [T,K], ids [T,K])."""
+    vals, ids = torch.topk(logits.float(), topk, dim=-1)
+    return torch.softmax(vals, dim=-1), ids.to(torch.int32)

@@ -39,6 +39,10 @@ class ForwardContext:
     # graph-replay path: persistent device slot buffer (all rows are
     # initialized decode steps; padding rows point at the dummy slot)
     ssm_slots_dev: Optional[object] = None
+    # device copies of ssm_slots (int64) / ssm_has_init (int32) for the
+    # ragged state kernels (causal_conv_silu, delta_rule_varlen)
+    ssm_slots_t: Optional[torch.Tensor] = None
+    ssm_has_init_t: Optional[torch.Tensor] = None
     # multimodal: rows of this batch whose embeddings come from the
     # vision tower (replaced after embed_tokens on the first stage)
     mm_rows: Optional[torch.Tensor] = None     # [N] long

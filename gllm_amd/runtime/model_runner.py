@@ -53,9 +53,18 @@ class ModelRunner:
             # can_replay). Requires the gfx950 GDN kernels.
             from gllm_amd import ops
             spec = self.model.ssm_spec
-            if not (cfg.device.startswith("cuda") and ops.has_kernels()
+            if spec.layers is None and not (
+                    cfg.device.startswith("cuda") and ops.has_kernels()
                     and spec.head_k_dim == 128 and spec.conv_kernel == 4):
                 cfg.use_graph = False
+        if not getattr(self.model, "supports_graph", True):
+            cfg.use_graph = False
+        if self.kv_dtype == torch.float32 and cfg.device.startswith("cuda"):
+            # float32 serving means true fp32 products (no TF32-class
+            # reduced-precision matrix mode)
+            torch.backends.cuda.matmul.allow_tf32 = False
+            torch.backends.cudnn.allow_tf32 = False
+            torch.set_float32_matmul_precision("highest")
         self.uses_mrope = bool(getattr(self.model, "uses_mrope", False))
         # mrope models capture with [3, B] position buffers (decode
         # positions are a per-seq scalar across all three sections);
@@ -115,7 +124,12 @@ class ModelRunner:
         self.ssm_snapshot_enabled = True
         if getattr(self.model, "ssm_spec", None) is not None:
             from gllm_amd.core.ssm import SSMPool
-            self.ssm_pool = SSMPool(self.model.ssm_spec, cfg.maxd + 64,
+            # one slot per live sequence plus the graph scratch slot;
+            # max_state_slots pins the pool (slots are then re-used as
+            # requests end), the default leaves headroom over maxd
+            n_slots = (cfg.max_state_slots + 1 if cfg.max_state_slots
+                       else cfg.maxd + 64)
+            self.ssm_pool = SSMPool(self.model.ssm_spec, n_slots,
                                     cfg.device, dtype=self.kv_dtype)
             self.memory_manager.free_hooks.append(self.ssm_pool.free)
             if isinstance(self.memory_manager, PrefixMemoryManager):
@@ -158,6 +172,14 @@ class ModelRunner:
             num_local_layers = self.model.num_local_layers
         # prefer the model's own attention geometry (configs name kv
         # heads differently, e.g. ChatGLM's multi_query_group_num)
+        shapes = getattr(self.model, "kv_layer_shapes", None)
+        if shapes is not None:
+            # heterogeneous stack: every cache-owning layer brings its
+            # own (kv_heads, k_dim, v_dim)
+            g0, dk0, dv0 = shapes[0] if shapes else (1, 8, 8)
+            return KVCacheSpec(len(shapes), g0, dk0, self.config.page_size,
+                               dtype_bytes=self.kv_dtype.itemsize,
+                               v_head_dim=dv0, layer_shapes=list(shapes))
         attn = getattr(self.model, "kv_geometry", None)
         if attn is not None:
             if len(attn) == 3:
@@ -268,6 +290,15 @@ class ModelRunner:
                   spec.head_dim)
         vshape = (num_pages, spec.page_size, spec.num_kv_heads,
                   spec.v_head_dim)
+        if spec.layer_shapes is not None:
+            self.k_caches = [torch.zeros(
+                (num_pages, spec.page_size, g, dk), dtype=self.kv_dtype,
+                device=self.device) for g, dk, _ in spec.layer_shapes]
+            self.v_caches = [torch.zeros(
+                (num_pages, spec.page_size, g, dv), dtype=self.kv_dtype,
+                device=self.device) for g, _, dv in spec.layer_shapes]
+            self.idx_caches = None
+            return
         self.k_caches = [torch.zeros(kshape, dtype=self.kv_dtype,
                                      device=self.device)
                          for _ in range(spec.num_layers)]
@@ -295,13 +326,9 @@ class ModelRunner:
         return self.model(input_ids, positions, fctx,
                           hidden_states=hidden_states, residual=residual)
 
-    @torch.no_grad()
-    def step_first_stage(self, batch: ScheduledBatch):
-        """Stage-0 forward. PP=1: returns sampled tokens. PP>1: returns
-        (hidden, residual, fctx) for the PP send."""
-        if self.graph_runner is not None and \
-                self.graph_runner.can_replay(batch):
-            return self.graph_runner.replay(batch)
+    def _forward_first_stage(self, batch: ScheduledBatch):
+        """Build the batch tensors, attach per-sequence state and run
+        this stage's layers. Returns (hidden, residual, fctx)."""
         tokens, fctx = self.builder.build(
             batch, self.k_caches, self.v_caches,
             need_logits=self.model.is_last_stage,
@@ -312,9 +339,34 @@ class ModelRunner:
         if fctx.has_placeholders:
             tokens = self.resolve_tokens(tokens)
         hidden, residual = self._stage_forward(tokens, fctx.positions, fctx)
+        return hidden, residual, fctx
+
+    @torch.no_grad()
+    def step_first_stage(self, batch: ScheduledBatch):
+        """Stage-0 forward. PP=1: returns sampled tokens. PP>1: returns
+        (hidden, residual, fctx) for the PP send."""
+        if self.graph_runner is not None and \
+                self.graph_runner.can_replay(batch):
+            return self.graph_runner.replay(batch)
+        hidden, residual, fctx = self._forward_first_stage(batch)
         if self.model.is_last_stage:
             return self._sample(batch, hidden, fctx)
         return hidden, residual, fctx
+
+    @torch.no_grad()
+    def step_logits(self, batch: ScheduledBatch, rows) -> torch.Tensor:
+        """The same forward as ``step_first_stage`` (batch builder, KV
+        pages, state slots, kernels) but instead of sampling it returns
+        the fp32 logits of the flat batch rows ``rows`` (row r of item i
+        is query_start_loc[i] + r). Used to replay token traces and to
+        score given continuations; PP=1 only."""
+        assert self.model.is_first_stage and self.model.is_last_stage
+        hidden, _, fctx = self._forward_first_stage(batch)
+        if len(rows) == 0:
+            return torch.empty(0, 0)
+        fctx.logits_indices = torch.as_tensor(
+            list(rows), dtype=torch.long, device=hidden.device)
+        return self.model.compute_logits(hidden, fctx).float()
 
     @torch.no_grad()
     def step_mid_stage(self, batch: ScheduledBatch, hidden, residual):
@@ -352,6 +404,14 @@ class ModelRunner:
             has_init.append(it.start > 0)
         fctx.ssm_slots = slots
         fctx.ssm_has_init = has_init
+        if getattr(self.model, "wants_state_tensors", False):
+            # ragged state kernels read slots / carried-state flags on
+            # the device
+            fctx.ssm_slots_t = torch.tensor(
+                slots, dtype=torch.long).to(self.device, non_blocking=True)
+            fctx.ssm_has_init_t = torch.tensor(
+                has_init, dtype=torch.int32).to(self.device,
+                                                non_blocking=True)
 
     def _attach_mm(self, batch, fctx) -> None:
         """Collect vision-embedding rows for this batch's prefill chunks

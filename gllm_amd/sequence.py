@@ -133,6 +133,14 @@ class Sequence:
     def is_finished(self) -> bool:
         return self.finish_reason is not None
 
+    def extend_prompt(self, token_ids: List[int]) -> None:
+        """Given (not sampled) tokens arriving after admission — a prompt
+        streamed in portions, or a continuation to be scored."""
+        self.token_ids.extend(token_ids)
+        self.prompt_len = len(self.token_ids)
+        self.raw_prompt_len = self.prompt_len
+        self.detok_offset = self.prompt_len
+
     # ---- decoding-loop transitions ----
     def append_token(self, token_id: int) -> None:
         self.token_ids.append(token_id)

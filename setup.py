@@ -1,9 +1,19 @@
-"""Build the in-tree gfx950 HIP kernel extension.
+"""Build the in-tree gfx950 HIP kernel extensions.
 
     PYTORCH_ROCM_ARCH=gfx950 python setup.py build_ext --inplace
 
-The .so lands next to the package (gllm_amd/_kernels*.so) so it travels
-with repo snapshots (gpurun) without a site-packages install.
+Two extension modules land next to the package so they travel with
+repo snapshots without a site-packages install:
+
+* ``gllm_amd._kernels``      every kernel family of the framework
+* ``gllm_amd._kernels_seq``  the dtype-generic sequence-mixer kernels
+  (layer norm over an fp32 residual, windowed sink attention, varlen
+  gated delta rule) plus the grouped MoE GEMM they are served with —
+  the only native code a Sudevik-style model needs, so a fresh
+  checkout can serve one after compiling five files instead of
+  fifteen.
+
+``GLLM_EXT=seq`` (or ``core``) restricts the build to one module.
 """
 
 import os
@@ -15,33 +25,39 @@ from torch.utils.cpp_extension import BuildExtension, CUDAExtension
 
 CSRC = os.path.join("gllm_amd", "ops", "csrc")
 
-ext = CUDAExtension(
-    name="gllm_amd._kernels",
-    sources=[
-        os.path.join(CSRC, "bindings.cpp"),
-        os.path.join(CSRC, "norm.hip"),
-        os.path.join(CSRC, "elementwise.hip"),
-        os.path.join(CSRC, "attention_decode.hip"),
-        os.path.join(CSRC, "attention_prefill.hip"),
-        os.path.join(CSRC, "attention_mla.hip"),
-        os.path.join(CSRC, "moe.hip"),
-        os.path.join(CSRC, "fp8.hip"),
-        os.path.join(CSRC, "gdn.hip"),
-        os.path.join(CSRC, "int4.hip"),
-        os.path.join(CSRC, "skinny_gemm.hip"),
-        os.path.join(CSRC, "sampling.hip"),
-        os.path.join(CSRC, "custom_ar.hip"),
-    ],
-    extra_compile_args={
-        "cxx": ["-O3", "-std=c++17"],
-        "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950"],
-    },
-)
+# -packed-fp32-ops: keep hipcc from forming v_pk_*_f32 out of scalar
+# float code (those forms have produced silent wrong results on gfx950)
+HIP_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+CXX_FLAGS = ["-O3", "-std=c++17"]
+
+SEQ_SOURCES = ["bindings_seq.cpp", "layernorm.hip", "attention_window.hip",
+               "delta_rule.hip", "moe.hip", "elementwise.hip"]
+CORE_SOURCES = ["bindings.cpp", "norm.hip", "elementwise.hip",
+                "attention_decode.hip", "attention_prefill.hip",
+                "attention_mla.hip", "moe.hip", "fp8.hip", "gdn.hip",
+                "int4.hip", "skinny_gemm.hip", "sampling.hip",
+                "custom_ar.hip"]
+
+
+def _ext(name, sources):
+    return CUDAExtension(
+        name=name,
+        sources=[os.path.join(CSRC, s) for s in sources],
+        extra_compile_args={"cxx": CXX_FLAGS, "nvcc": HIP_FLAGS})
+
+
+which = os.environ.get("GLLM_EXT", "all")
+exts = []
+if which in ("all", "core"):
+    exts.append(_ext("gllm_amd._kernels", CORE_SOURCES))
+if which in ("all", "seq"):
+    exts.append(_ext("gllm_amd._kernels_seq", SEQ_SOURCES))
 
 setup(
     name="gllm_amd",
     version="0.1.0",
     packages=["gllm_amd"],
-    ext_modules=[ext],
+    ext_modules=exts,
     cmdclass={"build_ext": BuildExtension},
 )
