@@ -185,6 +185,147 @@ MODELS = {
 }
 
 
+# ---------------------------------------------------------------------
+# --mixer-compare: Sudevik (windowed sink attention + gated delta rule +
+# routed experts, fp32 residual) beside the closest existing family
+# (Qwen3-Next-style hybrid GDN + gated attention + MoE) at equal layer
+# sizes, random weights. Prefill and decode tokens/s through the same
+# scripted engine path (scheduler pages -> batch builder -> kernels).
+COMPARE_SIZES = {
+    # name: width, attn (heads, kv, dim), delta (heads, kv, dk, dv),
+    #       experts, top, ff, layers
+    "w2048": dict(width=2048, attn=(16, 2, 128), delta=(16, 8, 128, 128),
+                  experts=32, top=4, ff=512, layers=8),
+    "w1024": dict(width=1024, attn=(16, 4, 64), delta=(8, 4, 128, 128),
+                  experts=16, top=2, ff=512, layers=8),
+}
+
+
+def sudevik_config(sz, vocab=32000, window=4096, keep=4):
+    H, G, D = sz["attn"]
+    dh, dg, dk, dv = sz["delta"]
+    mlp = {"kind": "moe", "expert": {"ff": sz["ff"]},
+           "router": {"experts": sz["experts"], "top": sz["top"]}}
+    layers = []
+    for i in range(sz["layers"]):
+        if (i + 1) % 4 == 0:
+            layers.append({"type": "attention", "mlp": mlp, "mixer": {
+                "heads": H, "kv_heads": G, "dim": D, "vdim": D,
+                "scale": D ** -0.5,
+                "mask": {"size": window, "keep_first": keep},
+                "rot": {"dims": D // 4, "base": 1000000.0}}})
+        else:
+            layers.append({"type": "delta", "mlp": mlp, "mixer": {
+                "heads": dh, "kv_heads": dg, "dim": dk, "vdim": dv,
+                "conv": 4}})
+    return {"architecture": "Sudevik", "layers": layers,
+            "norm": {"eps": 1e-5}, "vocab": vocab, "vocab_size": vocab,
+            "width": sz["width"]}
+
+
+def hybrid_gdn_config(sz, vocab=32000):
+    H, G, D = sz["attn"]
+    dh, dg, dk, dv = sz["delta"]
+    return {**QWEN3_NEXT_9B, "hidden_size": sz["width"],
+            "num_hidden_layers": sz["layers"], "num_attention_heads": H,
+            "num_key_value_heads": G, "head_dim": D,
+            "linear_num_value_heads": dh, "linear_num_key_heads": dg,
+            "linear_key_head_dim": dk, "linear_value_head_dim": dv,
+            "attn_output_gate": True, "num_experts": sz["experts"],
+            "num_experts_per_tok": sz["top"],
+            "moe_intermediate_size": sz["ff"],
+            "shared_expert_intermediate_size": 0, "norm_topk_prob": True,
+            "vocab_size": vocab}
+
+
+def mixer_compare(args):
+    from gllm_amd.config import EngineConfig
+    from gllm_amd.engine.llm import LLM
+    use_gpu = torch.cuda.is_available()
+    device = "cuda:0" if use_gpu else "cpu"
+    g = torch.Generator().manual_seed(7)
+    P = args.prompt_len
+    for size_name in args.compare_sizes.split(","):
+        sz = COMPARE_SIZES[size_name]
+        for fam, cfg_json in (("sudevik", sudevik_config(sz)),
+                              ("hybrid-gdn", hybrid_gdn_config(sz))):
+            cfg = EngineConfig(
+                model=write_model_dir(cfg_json), load_format="dummy",
+                dtype="bfloat16" if use_gpu else "float32", device=device,
+                page_size=16, maxp=1 << 20, maxd=1024, use_graph=False,
+                enable_overlap=False, enable_prefix_caching=False)
+            decode_bs = [int(x) for x in args.compare_decode.split(",")]
+            pages = (max(decode_bs + [args.compare_prefill_batch])
+                     * (P + 64 + 16) // 16 + 2)
+            llm = LLM(config=cfg, num_pages_override=pages)
+            llm.scheduler.log = False
+            sched, runner = llm.scheduler, llm.runner
+            vocab = cfg_json["vocab_size"]
+
+            def sync():
+                if use_gpu:
+                    torch.cuda.synchronize()
+
+            def prefill(B):
+                seqs = [llm.allocate_seq(torch.randint(
+                    1, vocab - 1, (P,), generator=g).tolist())
+                    for _ in range(B)]
+                sync()
+                t0 = time.time()
+                batch = sched.schedule_scripted([(s, P) for s in seqs])
+                runner.step_logits(batch, [P * (i + 1) - 1
+                                           for i in range(B)])
+                sched.commit_scripted(batch)
+                sync()
+                return seqs, time.time() - t0
+
+            def release(seqs):
+                for s in seqs:
+                    sched.release_scripted(s)
+                    llm.seq_id_alloc.free(s.seq_id)
+
+            B = args.compare_prefill_batch
+            release(prefill(B)[0])            # warmup
+            times = []
+            for _ in range(3):
+                seqs, dt = prefill(B)
+                times.append(dt)
+                release(seqs)
+            dt = sorted(times)[1]
+            print(json.dumps({"compare": size_name, "model": fam,
+                              "phase": "prefill", "batch": B,
+                              "prompt_len": P,
+                              "tokens_per_s": round(B * P / dt, 1),
+                              "ms": round(dt * 1000, 2)}), flush=True)
+            for B in decode_bs:
+                seqs, _ = prefill(B)
+
+                def step():
+                    for s in seqs:
+                        s.extend_prompt([5])
+                    batch = sched.schedule_scripted([(s, 1) for s in seqs])
+                    runner.step_logits(batch, list(range(B)))
+                    sched.commit_scripted(batch)
+
+                for _ in range(4):
+                    step()
+                sync()
+                t0 = time.time()
+                for _ in range(args.compare_steps):
+                    step()
+                sync()
+                dt = (time.time() - t0) / args.compare_steps
+                release(seqs)
+                print(json.dumps({"compare": size_name, "model": fam,
+                                  "phase": "decode", "batch": B,
+                                  "context": P,
+                                  "tokens_per_s": round(B / dt, 1),
+                                  "ms": round(dt * 1000, 3)}), flush=True)
+            del llm, sched, runner
+            if use_gpu:
+                torch.cuda.empty_cache()
+
+
 def write_model_dir(cfg_json):
     d = tempfile.mkdtemp(prefix="bench_model_")
     with open(os.path.join(d, "config.json"), "w") as f:
@@ -219,7 +360,18 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-overlap", action="store_true")
     ap.add_argument("--max-graph-bs", type=int, default=512)
+    ap.add_argument("--mixer-compare", action="store_true",
+                    help="instead of the flagship workload: Sudevik vs "
+                         "the hybrid-GDN family at equal layer sizes, "
+                         "prefill and decode tokens/s (one JSON line per "
+                         "case)")
+    ap.add_argument("--compare-sizes", type=str, default="w2048,w1024")
+    ap.add_argument("--compare-decode", type=str, default="1,32,128")
+    ap.add_argument("--compare-prefill-batch", type=int, default=4)
+    ap.add_argument("--compare-steps", type=int, default=16)
     args = ap.parse_args()
+    if args.mixer_compare:
+        return mixer_compare(args)
 
     world = int(os.environ.get("WORLD_SIZE", "1"))
     rank = int(os.environ.get("RANK", "0"))

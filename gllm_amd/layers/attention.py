@@ -127,4 +127,4 @@ class WindowAttention(nn.Module):
         return ops.window_attention(
             q, gate, k_cache, v_cache, fctx.block_table, fctx.seq_lens,
             fctx.query_start_loc, self.scale, self.window,
-            self.keep_first, self.sink)
+            self.keep_first, self.sink, fctx.max_query_len)

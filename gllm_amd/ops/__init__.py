@@ -784,15 +784,28 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
 
 def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
                      query_start_loc, scale, window=0, keep_first=0,
-                     sink=False) -> torch.Tensor:
+                     sink=False, max_query_len=0) -> torch.Tensor:
     """Ragged paged attention over K [pages, page, G, D] / V [.., Dv]:
     sliding window with kept first tokens, optional softmax sink (+1 in
-    the denominator) and fused sigmoid output gate. Returns [T, H*Dv]."""
+    the denominator) and fused sigmoid output gate. Returns [T, H*Dv].
+
+    Batches that hold prompt portions (``max_query_len`` > 1) in bf16
+    with D == Dv in {64, 128} run the MFMA tile kernel shared with
+    paged_attention (128 query rows per workgroup, K/V streamed through
+    LDS); decode-only batches, fp32 and every other head geometry run
+    the generic one-workgroup-per-(token, head) kernel."""
     if q.is_cuda:
         T = q.shape[0]
-        H = q.shape[1] // k_cache.shape[3]
-        out = torch.empty(T, H * v_cache.shape[3], dtype=q.dtype,
-                          device=q.device)
+        D, Dv = k_cache.shape[3], v_cache.shape[3]
+        H = q.shape[1] // D
+        out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+        if (max_query_len > 1 and q.dtype == torch.bfloat16 and D == Dv
+                and D in (64, 128)):
+            _seq_kernels().window_attention_mfma(
+                out, q, gate, k_cache, v_cache, block_table, seq_lens,
+                query_start_loc, max_query_len, scale, window, keep_first,
+                sink)
+            return out
         _seq_kernels().window_attention(
             out, q, gate, k_cache, v_cache, block_table, seq_lens,
             query_start_loc, scale, window, keep_first, sink)

@@ -50,7 +50,13 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
     const int *__restrict__ seq_lens,            // [B]
     const int *__restrict__ qsl,                 // [B+1]
     int max_pages, int page_size, int Hq, int num_kv_heads, float scale,
-    long q_stride, int window) {
+    long q_stride, int window,
+    // windowed-sink extensions (0 / 0 / nullptr = plain causal softmax):
+    // keys j < keep_first stay visible outside the window; sink adds a
+    // score-0, value-less key to the softmax (denominator 1 + sum exp);
+    // gate multiplies the output by sigmoid(gate[t, h*D + d])
+    int keep_first, int sink, const __hip_bfloat16 *__restrict__ gate,
+    long gate_stride) {
   const int tile = blockIdx.x;
   const int b = blockIdx.y;
   const int h = blockIdx.z;
@@ -95,7 +101,11 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
 
   float m_run[4], l_run[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) { m_run[r] = -INFINITY; l_run[r] = 0.f; }
+  for (int r = 0; r < 4; ++r) {
+    // the sink enters as an already-seen key of score 0
+    m_run[r] = sink ? 0.f : -INFINITY;
+    l_run[r] = sink ? 1.f : 0.f;
+  }
   mfma_f4 o_acc[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) o_acc[nt] = mfma_f4{0, 0, 0, 0};
@@ -128,15 +138,23 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
     }
   };
 
-  const int nkt = (kv_max - kv_lo + BKV - 1) / BKV;
+  // kept-first tiles [0, min(keep_first, kv_lo)) come before the
+  // window tiles; kv_lo is a BKV multiple, so the two never overlap
+  const int n_keep =
+      (keep_first > 0 && kv_lo > 0)
+          ? (min(keep_first, kv_lo) + BKV - 1) / BKV : 0;
+  const int nkt = n_keep + (kv_max - kv_lo + BKV - 1) / BKV;
+  auto tile_kv0 = [&](int t) {
+    return t < n_keep ? t * BKV : kv_lo + (t - n_keep) * BKV;
+  };
   const int pre = min(RING - 1, nkt);
-  for (int t = 0; t < pre; ++t) stage(kv_lo + t * BKV, t % RING);
+  for (int t = 0; t < pre; ++t) stage(tile_kv0(t), t % RING);
 
   for (int kt_i = 0; kt_i < nkt; ++kt_i) {
-    const int kv0 = kv_lo + kt_i * BKV;
+    const int kv0 = tile_kv0(kt_i);
     const int slot = kt_i % RING;
     if (kt_i + RING - 1 < nkt)
-      stage(kv_lo + (kt_i + RING - 1) * BKV, (kt_i + RING - 1) % RING);
+      stage(tile_kv0(kt_i + RING - 1), (kt_i + RING - 1) % RING);
     const int ahead = min(nkt - 1 - kt_i, RING - 1);
     if (ahead >= 1) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(GL_PER_WAVE) : "memory");
@@ -172,6 +190,7 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
     // window cut) skip the per-element mask lanes entirely
     const int qpos_min = past + tile * BQ + wave * 16;
     const bool full_tile =
+        kt_i >= n_keep &&
         qrow_valid && (tile * BQ + wave * 16 + 15 < q_len) &&
         (kv0 + BKV - 1 <= qpos_min) && (kv0 + BKV <= seq_len) &&
         (window <= 0 || kv0 > qpos_min + 15 - window);
@@ -196,7 +215,8 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
           float s = s_frag[f][r] * scale;
           if (qrow >= q_len || kvp > qpos || kvp >= seq_len)
             s = -INFINITY;
-          if (window > 0 && kvp <= qpos - window) s = -INFINITY;
+          if (window > 0 && kvp <= qpos - window && kvp >= keep_first)
+            s = -INFINITY;
           sv[f] = s;
           mx = fmaxf(mx, s);
         }
@@ -268,10 +288,56 @@ __global__ __launch_bounds__(BLOCK, 1) void paged_prefill_kernel(
     if (qrow >= q_len) continue;
     const float inv_l = (l_run[r] > 0.f) ? 1.f / l_run[r] : 0.f;
     __hip_bfloat16 *op = out + ((long)(q_start + qrow) * Hq + h) * D;
+    if (gate != nullptr) {
+      const __hip_bfloat16 *gp =
+          gate + (long)(q_start + qrow) * gate_stride + (long)h * D;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const float z = __bfloat162float(gp[nt * 16 + l16]);
+        op[nt * 16 + l16] = __float2bfloat16(
+            o_acc[nt][r] * inv_l / (1.f + __expf(-z)));
+      }
+      continue;
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
       op[nt * 16 + l16] = __float2bfloat16(o_acc[nt][r] * inv_l);
   }
+}
+
+}  // namespace
+
+namespace {
+
+void launch_prefill(torch::Tensor &out, torch::Tensor &q, int Hq, int D,
+                    long q_stride, torch::Tensor &k_cache,
+                    torch::Tensor &v_cache, torch::Tensor &block_table,
+                    torch::Tensor &seq_lens, torch::Tensor &query_start_loc,
+                    long max_query_len, double scale, long window,
+                    long keep_first, bool sink, const void *gate,
+                    long gate_stride) {
+  const int Hkv = k_cache.size(2);
+  const int B = seq_lens.size(0);
+  const int q_tiles = (int)((max_query_len + BQ - 1) / BQ);
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(DV)                                                              \
+  hipLaunchKernelGGL((paged_prefill_kernel<DV>), dim3(q_tiles, B, Hq),       \
+                     dim3(BLOCK), 0, stream,                                 \
+                     (__hip_bfloat16 *)out.data_ptr(),                       \
+                     (const __hip_bfloat16 *)q.data_ptr(),                   \
+                     (const __hip_bfloat16 *)k_cache.data_ptr(),             \
+                     (const __hip_bfloat16 *)v_cache.data_ptr(),             \
+                     block_table.data_ptr<int>(), seq_lens.data_ptr<int>(),  \
+                     query_start_loc.data_ptr<int>(),                        \
+                     (int)block_table.stride(0), (int)k_cache.size(1), Hq,   \
+                     Hkv, (float)scale, q_stride, (int)window,               \
+                     (int)keep_first, sink ? 1 : 0,                          \
+                     (const __hip_bfloat16 *)gate, gate_stride)
+  if (D == 128) RUN(128);
+  else if (D == 64) RUN(64);
+  else TORCH_CHECK(false, "prefill attn: head_dim ", D, " unsupported");
+#undef RUN
+  HIP_CHECK_KERNEL();
 }
 
 }  // namespace
@@ -287,40 +353,52 @@ void paged_attention_prefill(torch::Tensor out, torch::Tensor q,
   TORCH_CHECK(out.is_contiguous());
   TORCH_CHECK(q.stride(2) == 1 && q.stride(1) == q.size(2),
               "q per-token row must be contiguous");
-  const int D = q.size(2);
-  const int Hq = q.size(1);
-  const int Hkv = k_cache.size(2);
-  const int B = seq_lens.size(0);
+  if (q.size(0) == 0) return;
+  launch_prefill(out, q, q.size(1), q.size(2), q.stride(0), k_cache, v_cache,
+                 block_table, seq_lens, query_start_loc, max_query_len,
+                 scale, sliding_window, 0, false, nullptr, 0);
+}
+
+// Windowed-sink form of the same MFMA kernel: q [T, H*D] (row-strided
+// view allowed), bf16, D == Dv in {64, 128}. Callers route every other
+// shape / dtype to the generic window_attention kernel.
+void window_attention_mfma(torch::Tensor out, torch::Tensor q,
+                           c10::optional<torch::Tensor> gate,
+                           torch::Tensor k_cache, torch::Tensor v_cache,
+                           torch::Tensor block_table, torch::Tensor seq_lens,
+                           torch::Tensor query_start_loc, long max_query_len,
+                           double scale, long window, long keep_first,
+                           bool sink) {
   const long T = q.size(0);
   if (T == 0) return;
-  const int q_tiles = (int)((max_query_len + BQ - 1) / BQ);
-  auto stream = at::cuda::getCurrentCUDAStream();
-  if (D == 128) {
-    hipLaunchKernelGGL((paged_prefill_kernel<128>),
-                       dim3(q_tiles, B, Hq), dim3(BLOCK), 0, stream,
-                       (__hip_bfloat16 *)out.data_ptr(),
-                       (const __hip_bfloat16 *)q.data_ptr(),
-                       (const __hip_bfloat16 *)k_cache.data_ptr(),
-                       (const __hip_bfloat16 *)v_cache.data_ptr(),
-                       block_table.data_ptr<int>(), seq_lens.data_ptr<int>(),
-                       query_start_loc.data_ptr<int>(),
-                       (int)block_table.size(1), (int)k_cache.size(1), Hq,
-                       Hkv, (float)scale, q.stride(0),
-                       (int)sliding_window);
-  } else if (D == 64) {
-    hipLaunchKernelGGL((paged_prefill_kernel<64>),
-                       dim3(q_tiles, B, Hq), dim3(BLOCK), 0, stream,
-                       (__hip_bfloat16 *)out.data_ptr(),
-                       (const __hip_bfloat16 *)q.data_ptr(),
-                       (const __hip_bfloat16 *)k_cache.data_ptr(),
-                       (const __hip_bfloat16 *)v_cache.data_ptr(),
-                       block_table.data_ptr<int>(), seq_lens.data_ptr<int>(),
-                       query_start_loc.data_ptr<int>(),
-                       (int)block_table.size(1), (int)k_cache.size(1), Hq,
-                       Hkv, (float)scale, q.stride(0),
-                       (int)sliding_window);
-  } else {
-    TORCH_CHECK(false, "prefill attn: head_dim ", D, " unsupported");
+  const int D = k_cache.size(3);
+  TORCH_CHECK(q.scalar_type() == at::kBFloat16 &&
+              k_cache.scalar_type() == at::kBFloat16 &&
+              v_cache.scalar_type() == at::kBFloat16);
+  TORCH_CHECK(v_cache.size(3) == D && (D == 64 || D == 128),
+              "window_attention_mfma: D == Dv in {64, 128}");
+  TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q.size(1) % D == 0);
+  const int H = q.size(1) / D;
+  TORCH_CHECK(H % k_cache.size(2) == 0);
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous());
+  TORCH_CHECK(out.is_contiguous() && out.scalar_type() == at::kBFloat16 &&
+              out.numel() == T * H * D);
+  TORCH_CHECK(block_table.scalar_type() == at::kInt &&
+              block_table.stride(1) == 1 &&
+              seq_lens.scalar_type() == at::kInt &&
+              query_start_loc.scalar_type() == at::kInt);
+  TORCH_CHECK(query_start_loc.numel() >= seq_lens.numel() + 1 &&
+              block_table.size(0) >= seq_lens.numel());
+  const void *gp = nullptr;
+  long gs = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->dim() == 2 && gate->stride(1) == 1 &&
+                gate->size(0) == T && gate->size(1) == (long)H * D &&
+                gate->scalar_type() == at::kBFloat16);
+    gp = gate->data_ptr();
+    gs = gate->stride(0);
   }
-  HIP_CHECK_KERNEL();
+  launch_prefill(out, q, H, D, q.stride(0), k_cache, v_cache, block_table,
+                 seq_lens, query_start_loc, max_query_len, scale, window,
+                 keep_first, sink, gp, gs);
 }

@@ -147,7 +147,23 @@ __global__ __launch_bounds__(ATT_BLOCK) void window_attention_kernel(
       rows[tid] = row;
       const T *kr = k_cache + (row * G + g) * D;
       float dot = 0.f;
-      for (int d = 0; d < D; ++d) dot += qs[d] * ScalarOps<T>::to_f32(kr[d]);
+      if (sizeof(T) == 2 && D % 8 == 0) {  // 16 B loads, rows 16 B aligned
+        for (int d = 0; d < D; d += 8) {
+          float kf[8];
+          unpack8<T>(*reinterpret_cast<const shortx8 *>(kr + d), kf);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dot += qs[d + e] * kf[e];
+        }
+      } else if (sizeof(T) == 4 && D % 4 == 0) {
+        for (int d = 0; d < D; d += 4) {
+          const floatx4 kf = *reinterpret_cast<const floatx4 *>(kr + d);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dot += qs[d + e] * kf[e];
+        }
+      } else {
+        for (int d = 0; d < D; ++d)
+          dot += qs[d] * ScalarOps<T>::to_f32(kr[d]);
+      }
       s = dot * scale;
     }
     // tile max -> new running max

@@ -27,6 +27,13 @@ void paged_attention_prefill(torch::Tensor out, torch::Tensor q,
                              torch::Tensor query_start_loc,
                              long max_query_len, double scale,
                              long sliding_window);
+void window_attention_mfma(torch::Tensor out, torch::Tensor q,
+                           c10::optional<torch::Tensor> gate,
+                           torch::Tensor k_cache, torch::Tensor v_cache,
+                           torch::Tensor block_table, torch::Tensor seq_lens,
+                           torch::Tensor query_start_loc, long max_query_len,
+                           double scale, long window, long keep_first,
+                           bool sink);
 void mla_paged_attention(torch::Tensor out, torch::Tensor q,
                          torch::Tensor k_cache, torch::Tensor block_table,
                          torch::Tensor seq_lens,
@@ -106,6 +113,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "split-KV paged decode attention");
   m.def("paged_attention_prefill", &paged_attention_prefill,
         "varlen MFMA paged prefill attention");
+  m.def("window_attention_mfma", &window_attention_mfma,
+        "prefill MFMA kernel with window + kept first tokens + sink + gate");
   m.def("skinny_gemm", &skinny_gemm,
         "decode-regime weight-streaming GEMM (M<=256)");
   m.def("mla_paged_attention", &mla_paged_attention,

@@ -183,13 +183,22 @@ def rel_err(got, want):
 
 
 def check_against_oracle(cfg, weights, got, prompts, tol):
-    worst = 0.0
+    """fp32: every position within tol. bf16: the 16-bit rounding of a
+    router's input can flip a close top-k call, which moves that
+    position's logits by far more than rounding does; allow a few such
+    positions (a wrong mechanism moves most of them)."""
+    worst, refs = 0.0, {}
     for rid, rows in got.items():
-        ref = oracle.forward(cfg, weights, prompts[rid.split("#")[0]]).numpy()
-        for pos, logits in rows.items():
-            e = rel_err(logits, ref[pos])
-            worst = max(worst, e)
-            assert e < tol, (rid, pos, e)
+        key = tuple(prompts[rid.split("#")[0]])
+        if key not in refs:
+            refs[key] = oracle.forward(cfg, weights, list(key)).numpy()
+        errs = {pos: rel_err(lg, refs[key][pos]) for pos, lg in rows.items()}
+        over = {p: e for p, e in errs.items() if not e < tol}
+        if tol < 1e-2:
+            assert not over, (rid, over)
+        else:
+            assert len(over) <= max(1, len(errs) // 16), (rid, over)
+        worst = max(worst, max(errs.values()))
     return worst
 
 
@@ -305,8 +314,9 @@ def test_mixed_batches_recycle_pages_and_slots(device, dtype):
     check_against_oracle(cfg, w, got, P, TOL[dtype])
 
 
+@pytest.mark.parametrize("dims", [(8, 6), (64, 64)], ids=["d8", "d64"])
 @pytest.mark.parametrize("device,dtype", DEVICES)
-def test_window_and_kept_edges_stand_out(device, dtype):
+def test_window_and_kept_edges_stand_out(device, dtype, dims):
     """ops.window_attention with one planted key whose score towers over
     the rest: the output equals that key's value exactly when the key is
     visible — just inside / outside the window, the last kept token /
@@ -314,7 +324,8 @@ def test_window_and_kept_edges_stand_out(device, dtype):
     — for a query inside a prompt portion and for a decoded token."""
     from gllm_amd import ops
     tdt = getattr(torch, dtype)
-    page, G, H, D, Dv = 16, 2, 4, 8, 6
+    page, G, H = 16, 2, 4
+    D, Dv = dims   # (64, 64) in bf16 with a portion takes the MFMA kernel
     W, keep, L = 40, 3, 300
     g = torch.Generator().manual_seed(7)
     npages = 64
@@ -339,7 +350,7 @@ def test_window_and_kept_edges_stand_out(device, dtype):
             kc.to(tdt).to(device), vc.to(tdt).to(device), bt,
             torch.tensor([i + 1], dtype=torch.int32, device=device),
             torch.tensor([0, q_len], dtype=torch.int32, device=device),
-            1.0, W, keep, True)
+            1.0, W, keep, True, q_len)
         return out[-1].float().cpu()
 
     for q_len in (1, 23):
@@ -354,7 +365,6 @@ def test_window_and_kept_edges_stand_out(device, dtype):
                 else:
                     assert o.abs().max() < 10.0, (q_len, i, j, o)
     # plain causal (no window): a key hundreds back is seen
-    k_far = run  # noqa: F841  (window 0 case below)
     k = 0.05 * torch.randn(L, G, D, generator=g)
     v = torch.randn(L, G, Dv, generator=g)
     k[5, :, 0] = 30.0
@@ -404,7 +414,7 @@ def test_sink_takes_its_share(device, dtype):
 def test_far_state_survives_long_decoding(device, dtype):
     """A delta-only model decoded token by token for 100 steps after a
     short prompt: the state carries the early tokens all the way."""
-    cfg = make_config([with_moe(delta(conv=4)), no_mlp(delta(
+    cfg = make_config([no_mlp(delta(conv=4)), no_mlp(delta(
         heads=2, kv_heads=1, dim=16, vdim=16, conv=2))], width=24, vocab=40)
     w = make_weights(cfg, 9)
     for i in range(2):  # slow decay, or 100 random steps forget the start
@@ -461,6 +471,7 @@ def test_greedy_generation_through_the_scheduler(device, dtype):
     outs = llm.generate(prompts, SamplingParams(
         temperature=0.0, max_tokens=12, ignore_eos=True))
     margin = 0.05 if dtype == "float32" else 0.5
+    checked = 0
     for p, o in zip(prompts, outs):
         seq = list(p)
         for tok in o.token_ids:
@@ -470,7 +481,8 @@ def test_greedy_generation_through_the_scheduler(device, dtype):
                 break  # a near-tie proves nothing either way
             assert tok == int(logits.argmax()), (len(seq), tok)
             seq.append(tok)
-        assert len(seq) > len(p)
+            checked += 1
+    assert checked >= 8
 
 
 def test_config_and_registry():
@@ -491,3 +503,110 @@ def test_config_and_registry():
                                                 (64, 4, 12, 8)]
     with pytest.raises(KeyError):
         model.load_weights([("l0.mix.nonsense", torch.zeros(1))])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("D,Dv,dtype", [
+    (64, 64, "bfloat16"), (128, 128, "bfloat16"), (64, 64, "float32"),
+    (24, 40, "bfloat16"), (16, 8, "float32"), (128, 64, "bfloat16")])
+@pytest.mark.parametrize("window,keep", [(50, 3), (0, 0), (130, 70)])
+def test_window_attention_kernels_match_reference(D, Dv, dtype, window,
+                                                  keep):
+    """Both GPU kernels (MFMA tiles for bf16 D == Dv in {64, 128} when a
+    portion is in the batch, the generic kernel otherwise) against the
+    torch reference of the same op on a ragged batch: portions with and
+    without a past beside single decode tokens, shuffled pages, gate."""
+    from gllm_amd import ops
+    from gllm_amd.ops import torch_ref
+    tdt = getattr(torch, dtype)
+    g = torch.Generator().manual_seed(D + Dv + window)
+    page, G, H = 16, 2, 6
+    geo = [(0, 200), (37, 1), (130, 77), (300, 1), (5, 2), (63, 129)]
+    lens = [p + n for p, n in geo]
+    npages = sum(-(-L // page) for L in lens) + 3
+    perm = torch.randperm(npages, generator=g).tolist()
+    maxp = max(-(-L // page) for L in lens)
+    bt = torch.zeros(len(geo), maxp, dtype=torch.int32)
+    for b, L in enumerate(lens):
+        n = -(-L // page)
+        bt[b, :n] = torch.tensor([perm.pop() for _ in range(n)])
+    kc = torch.randn(npages, page, G, D, generator=g).to(tdt)
+    vc = torch.randn(npages, page, G, Dv, generator=g).to(tdt)
+    T = sum(n for _, n in geo)
+    q = (torch.randn(T, H * D, generator=g) * 0.5).to(tdt)
+    gate = torch.randn(T, H * Dv, generator=g).to(tdt)
+    qsl = torch.tensor([0] + list(np.cumsum([n for _, n in geo])),
+                       dtype=torch.int32)
+    sl = torch.tensor(lens, dtype=torch.int32)
+    scale = D ** -0.5
+    for use_gate in (True, False):
+        for sink in (True, False):
+            gt = gate if use_gate else None
+            want = torch_ref.window_attention(
+                q.float(), None if gt is None else gt.float(), kc.float(),
+                vc.float(), bt, sl, qsl, scale, window, keep, sink)
+            for mql in (200, 1):
+                # mql == 1 forces the generic kernel on the same batch
+                got = ops.window_attention(
+                    q.cuda(), None if gt is None else gt.cuda(), kc.cuda(),
+                    vc.cuda(), bt.cuda(), sl.cuda(), qsl.cuda(), scale,
+                    window, keep, sink, mql).float().cpu()
+                tol = 2e-2 if dtype == "bfloat16" else 2e-5
+                err = (got - want).abs().max().item()
+                assert err < tol, (use_gate, sink, mql, err)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,Dk,Dv,taps", [
+    (4, 2, 128, 128, 4), (3, 1, 20, 5, 2), (2, 2, 64, 96, 3),
+    (8, 4, 32, 16, 1), (2, 1, 200, 72, 8)])
+def test_delta_rule_kernels_match_reference(H, G, Dk, Dv, taps, dtype):
+    """causal_conv_silu + delta_rule_varlen + rms_gate on the GPU against
+    the torch reference of the same ops: ragged batch (fresh portions,
+    continued portions, decode tokens), state slots out of order."""
+    from gllm_amd import ops
+    from gllm_amd.ops import gdn_ref
+    tdt = getattr(torch, dtype)
+    g = torch.Generator().manual_seed(H * Dk + Dv + taps)
+    geo = [(False, 70), (True, 1), (True, 9), (False, 2), (True, 1)]
+    slots = torch.tensor([3, 0, 5, 1, 4])
+    n_slots = 7
+    T = sum(n for _, n in geo)
+    C = 2 * G * Dk + H * Dv
+    qsl = torch.tensor([0] + list(np.cumsum([n for _, n in geo])),
+                       dtype=torch.int32)
+    init = torch.tensor([int(i) for i, _ in geo], dtype=torch.int32)
+    x = torch.randn(T, C + 7, generator=g).to(tdt)[:, 3:3 + C]  # a slice
+    w = (torch.randn(C, taps, generator=g) * 0.5).to(tdt)
+    cs = torch.randn(n_slots, C, max(taps - 1, 1), generator=g).to(tdt)
+    st = torch.randn(n_slots, H, Dk, Dv, generator=g) * 0.3
+    ab = torch.randn(T, 2 * H, generator=g).to(tdt)
+    A_log = torch.rand(H, generator=g) * 2 - 1.5
+    dtb = torch.randn(H, generator=g)
+    z = torch.randn(T, H * Dv, generator=g).to(tdt)
+    nw = (1 + 0.2 * torch.randn(Dv, generator=g)).to(tdt)
+
+    def run(dev):
+        cs_d, st_d = cs.clone().to(dev), st.clone().to(dev)
+        conv = ops.causal_conv_silu(x.to(dev), w.to(dev), cs_d,
+                                    slots.to(dev), init.to(dev),
+                                    qsl.to(dev))
+        gk = G * Dk
+        abd = ab.to(dev)
+        o = ops.delta_rule_varlen(
+            conv[:, :gk], conv[:, gk:2 * gk], conv[:, 2 * gk:],
+            abd[:, :H], abd[:, H:], A_log.to(dev), dtb.to(dev), st_d,
+            slots.to(dev), init.to(dev), qsl.to(dev), Dk ** -0.5)
+        out = ops.rms_gate(o, z.to(dev), nw.to(dev), H, 1e-5, tdt)
+        return (conv.float().cpu(), o.cpu(), out.float().cpu(),
+                cs_d.float().cpu(), st_d.cpu())
+
+    want, got = run("cpu"), run("cuda")
+    tol = 3e-2 if dtype == "bfloat16" else 1e-4
+    for name, a, b in zip(("conv", "o", "out", "conv_state", "state"),
+                          want, got):
+        scale = max(1.0, a.abs().max().item())
+        assert (a - b).abs().max().item() < tol * scale, name
+    # untouched slots stay as they were
+    assert torch.equal(got[4][2], st[2]) and torch.equal(got[4][6], st[6])
