@@ -792,8 +792,9 @@ def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
     Batches that hold prompt portions (``max_query_len`` > 1) in bf16
     with D == Dv in {64, 128} run the MFMA tile kernel shared with
     paged_attention (128 query rows per workgroup, K/V streamed through
-    LDS); decode-only batches, fp32 and every other head geometry run
-    the generic one-workgroup-per-(token, head) kernel."""
+    LDS); decode-only bf16 batches with an instantiated (D, GQA ratio)
+    run the split-KV decode kernels; fp32 and every other head geometry
+    run the generic one-workgroup-per-(token, head) kernel."""
     if q.is_cuda:
         T = q.shape[0]
         D, Dv = k_cache.shape[3], v_cache.shape[3]
@@ -805,6 +806,13 @@ def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
                 out, q, gate, k_cache, v_cache, block_table, seq_lens,
                 query_start_loc, max_query_len, scale, window, keep_first,
                 sink)
+            return out
+        if (max_query_len == 1 and q.dtype == torch.bfloat16 and D == Dv
+                and _seq_kernels().window_attention_decode(
+                    out, q, gate, k_cache, v_cache, block_table, seq_lens,
+                    scale, window, keep_first, sink)):
+            # decode-only batch on the split-KV kernels shared with
+            # paged_attention (one workgroup per GQA group and KV split)
             return out
         _seq_kernels().window_attention(
             out, q, gate, k_cache, v_cache, block_table, seq_lens,

@@ -34,7 +34,7 @@ __global__ __launch_bounds__(BLOCK) void paged_decode_kernel(
     const int *__restrict__ block_table,  // [B, max_pages]
     const int *__restrict__ seq_lens,     // [B]
     int max_pages, int page_size, int num_kv_heads, float scale,
-    int num_splits, long q_stride, int window) {
+    int num_splits, long q_stride, int window, int keep_first) {
   const int b = blockIdx.x;
   const int kvh = blockIdx.y;
   const int split = blockIdx.z;
@@ -47,8 +47,13 @@ __global__ __launch_bounds__(BLOCK) void paged_decode_kernel(
   // split token range (page-aligned chunks not required; rows are
   // addressed per token through the block table)
   const int split_len = (visible + num_splits - 1) / num_splits;
-  const int t0 = w_begin + split * split_len;
-  const int t1 = min(t0 + split_len, seq_len);
+  // split == num_splits (launched only when keep_first > 0) is the
+  // kept-first segment [0, min(keep_first, w_begin)): tokens that stay
+  // visible outside the window; its partial merges like any other
+  const bool kept = split == num_splits;
+  const int t0 = kept ? 0 : w_begin + split * split_len;
+  const int t1 = kept ? min(keep_first, w_begin)
+                      : min(t0 + split_len, seq_len);
   const int lane_per_tok = D / 8;            // 16 lanes for D=128
   const int toks_per_iter = BLOCK / lane_per_tok;
 
@@ -258,7 +263,7 @@ __global__ __launch_bounds__(BLOCK) void paged_decode_mfma_kernel(
     const __hip_bfloat16 *__restrict__ v_cache,
     const int *__restrict__ block_table, const int *__restrict__ seq_lens,
     int max_pages, int page_size, int num_kv_heads, float scale,
-    int num_splits, long q_stride, int window) {
+    int num_splits, long q_stride, int window, int keep_first) {
   constexpr int D = 128;
   constexpr int CK = 64;            // kv tokens per chunk
   const int b = blockIdx.x;
@@ -269,8 +274,13 @@ __global__ __launch_bounds__(BLOCK) void paged_decode_mfma_kernel(
   const int w_begin = (window > 0) ? max(0, seq_len - window) : 0;
   const int visible = seq_len - w_begin;
   const int split_len = (visible + num_splits - 1) / num_splits;
-  const int t0 = w_begin + split * split_len;
-  const int t1 = min(t0 + split_len, seq_len);
+  // split == num_splits (launched only when keep_first > 0) is the
+  // kept-first segment [0, min(keep_first, w_begin)): tokens that stay
+  // visible outside the window; its partial merges like any other
+  const bool kept = split == num_splits;
+  const int t0 = kept ? 0 : w_begin + split * split_len;
+  const int t1 = kept ? min(keep_first, w_begin)
+                      : min(t0 + split_len, seq_len);
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -467,14 +477,16 @@ __global__ void decode_merge_kernel(
     __hip_bfloat16 *__restrict__ out,       // [B, Hq, D]
     const float *__restrict__ partial_out,  // [S, B, Hq, D]
     const float *__restrict__ partial_lse,  // [S, B, Hq]
-    int num_splits, int Hq) {
+    int num_splits, int Hq, int sink,
+    const __hip_bfloat16 *__restrict__ gate, long gate_stride) {
   const int b = blockIdx.x, h = blockIdx.y;
   const int d = threadIdx.x;
   const int B = gridDim.x;
-  float mx = -INFINITY;
+  // sink: one more "partial" with lse 0 and no value
+  float mx = sink ? 0.f : -INFINITY;
   for (int s = 0; s < num_splits; ++s)
     mx = fmaxf(mx, partial_lse[((long)s * B + b) * Hq + h]);
-  float denom = 0.f, o = 0.f;
+  float denom = sink ? __expf(-mx) : 0.f, o = 0.f;
   for (int s = 0; s < num_splits; ++s) {
     const float lse = partial_lse[((long)s * B + b) * Hq + h];
     if (lse == -INFINITY) continue;
@@ -482,8 +494,13 @@ __global__ void decode_merge_kernel(
     denom += w;
     o += w * partial_out[(((long)s * B + b) * Hq + h) * D + d];
   }
-  out[((long)b * Hq + h) * D + d] =
-      __float2bfloat16(denom > 0.f ? o / denom : 0.f);
+  float res = denom > 0.f ? o / denom : 0.f;
+  if (gate != nullptr) {
+    const float z =
+        __bfloat162float(gate[(long)b * gate_stride + (long)h * D + d]);
+    res *= 1.f / (1.f + __expf(-z));
+  }
+  out[((long)b * Hq + h) * D + d] = __float2bfloat16(res);
 }
 
 template <int D, int G>
@@ -491,10 +508,12 @@ void launch_decode(torch::Tensor &out, const torch::Tensor &q,
                    const torch::Tensor &k_cache, const torch::Tensor &v_cache,
                    const torch::Tensor &block_table,
                    const torch::Tensor &seq_lens, float scale,
-                   int max_seq_len, long q_stride, int window) {
+                   int max_seq_len, long q_stride, int window,
+                   int keep_first = 0, bool sink = false,
+                   const void *gate = nullptr, long gate_stride = 0) {
   const int B = q.size(0);
-  const int Hq = q.size(1);
   const int Hkv = k_cache.size(2);
+  const int Hq = Hkv * G;
   constexpr int CHUNK = 128;
   // split heuristic: enough workgroups to fill 256 CUs x 8 XCDs
   static int splits_env = [] {
@@ -508,8 +527,10 @@ void launch_decode(torch::Tensor &out, const torch::Tensor &q,
     splits *= 2;
   if (splits_env > 0) splits = splits_env;
   auto opts = q.options().dtype(at::kFloat);
-  auto partial = torch::empty({splits, B, Hq, D}, opts);
-  auto lse = torch::empty({splits, B, Hq}, opts);
+  // + 1: the kept-first segment of a windowed layer
+  const int zdim = splits + ((keep_first > 0 && window > 0) ? 1 : 0);
+  auto partial = torch::empty({zdim, B, Hq, D}, opts);
+  auto lse = torch::empty({zdim, B, Hq}, opts);
   auto stream = at::cuda::getCurrentCUDAStream();
   static int no_mfma = [] {
     const char *e = getenv("GLLM_DECODE_NO_MFMA");
@@ -517,31 +538,32 @@ void launch_decode(torch::Tensor &out, const torch::Tensor &q,
   }();
   if (D == 128 && G <= 16 && !no_mfma) {
     hipLaunchKernelGGL((paged_decode_mfma_kernel<G>),
-                       dim3(B, Hkv, splits), dim3(BLOCK), 0, stream,
+                       dim3(B, Hkv, zdim), dim3(BLOCK), 0, stream,
                        partial.data_ptr<float>(), lse.data_ptr<float>(),
                        (const __hip_bfloat16 *)q.data_ptr(),
                        (const __hip_bfloat16 *)k_cache.data_ptr(),
                        (const __hip_bfloat16 *)v_cache.data_ptr(),
                        block_table.data_ptr<int>(),
-                       seq_lens.data_ptr<int>(), (int)block_table.size(1),
+                       seq_lens.data_ptr<int>(), (int)block_table.stride(0),
                        (int)k_cache.size(1), Hkv, scale, splits, q_stride,
-                       window);
+                       window, keep_first);
   } else {
     hipLaunchKernelGGL((paged_decode_kernel<D, G, CHUNK>),
-                       dim3(B, Hkv, splits), dim3(BLOCK), 0, stream,
+                       dim3(B, Hkv, zdim), dim3(BLOCK), 0, stream,
                        partial.data_ptr<float>(), lse.data_ptr<float>(),
                        (const __hip_bfloat16 *)q.data_ptr(),
                        (const __hip_bfloat16 *)k_cache.data_ptr(),
                        (const __hip_bfloat16 *)v_cache.data_ptr(),
                        block_table.data_ptr<int>(), seq_lens.data_ptr<int>(),
-                       (int)block_table.size(1), (int)k_cache.size(1), Hkv,
-                       scale, splits, q_stride, window);
+                       (int)block_table.stride(0), (int)k_cache.size(1), Hkv,
+                       scale, splits, q_stride, window, keep_first);
   }
   HIP_CHECK_KERNEL();
   hipLaunchKernelGGL((decode_merge_kernel<D>), dim3(B, Hq), dim3(D), 0,
                      stream, (__hip_bfloat16 *)out.data_ptr(),
-                     partial.data_ptr<float>(), lse.data_ptr<float>(), splits,
-                     Hq);
+                     partial.data_ptr<float>(), lse.data_ptr<float>(), zdim,
+                     Hq, sink ? 1 : 0, (const __hip_bfloat16 *)gate,
+                     gate_stride);
   HIP_CHECK_KERNEL();
 }
 
@@ -577,4 +599,56 @@ void paged_attention_decode(torch::Tensor out, torch::Tensor q,
 #undef CASE
   TORCH_CHECK(false, "paged_attention_decode: unsupported head_dim=", D,
               " group=", G);
+}
+
+// Windowed-sink form of the split-KV decode kernels: one decode token per
+// sequence, q [B, H*D] (row-strided view allowed), bf16, D == Dv in
+// {64, 128} and a GQA ratio the kernels are instantiated for; returns
+// false (nothing launched) for any other geometry so the caller can take
+// the generic kernel.
+bool window_attention_decode(torch::Tensor out, torch::Tensor q,
+                             c10::optional<torch::Tensor> gate,
+                             torch::Tensor k_cache, torch::Tensor v_cache,
+                             torch::Tensor block_table,
+                             torch::Tensor seq_lens, double scale,
+                             long window, long keep_first, bool sink) {
+  const int B = q.size(0);
+  if (B == 0) return true;
+  const int D = k_cache.size(3);
+  const int Hkv = k_cache.size(2);
+  if (q.scalar_type() != at::kBFloat16 || v_cache.size(3) != D ||
+      q.dim() != 2 || q.size(1) % (D * Hkv) != 0)
+    return false;
+  const int G = q.size(1) / D / Hkv;
+  TORCH_CHECK(q.stride(1) == 1 && out.is_contiguous() &&
+              out.scalar_type() == at::kBFloat16 &&
+              out.numel() == (long)B * Hkv * G * D);
+  TORCH_CHECK(k_cache.scalar_type() == at::kBFloat16 &&
+              v_cache.scalar_type() == at::kBFloat16 &&
+              k_cache.is_contiguous() && v_cache.is_contiguous());
+  TORCH_CHECK(block_table.scalar_type() == at::kInt &&
+              block_table.stride(1) == 1 && block_table.size(0) >= B);
+  TORCH_CHECK(seq_lens.scalar_type() == at::kInt && seq_lens.numel() == B);
+  const void *gp = nullptr;
+  long gs = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->dim() == 2 && gate->stride(1) == 1 &&
+                gate->size(0) == B && gate->size(1) == q.size(1) &&
+                gate->scalar_type() == at::kBFloat16);
+    gp = gate->data_ptr();
+    gs = gate->stride(0);
+  }
+  const int max_seq = k_cache.size(0) * k_cache.size(1);
+#define CASE(DD, GG)                                                       \
+  if (D == DD && G == GG) {                                                \
+    launch_decode<DD, GG>(out, q, k_cache, v_cache, block_table, seq_lens, \
+                          (float)scale, max_seq, q.stride(0), (int)window, \
+                          (int)keep_first, sink, gp, gs);                  \
+    return true;                                                           \
+  }
+  CASE(128, 1) CASE(128, 2) CASE(128, 4) CASE(128, 5) CASE(128, 8)
+  CASE(64, 1) CASE(64, 2) CASE(64, 4) CASE(64, 8)
+  CASE(128, 16)
+#undef CASE
+  return false;
 }

@@ -34,6 +34,12 @@ void window_attention_mfma(torch::Tensor out, torch::Tensor q,
                            torch::Tensor query_start_loc, long max_query_len,
                            double scale, long window, long keep_first,
                            bool sink);
+bool window_attention_decode(torch::Tensor out, torch::Tensor q,
+                             c10::optional<torch::Tensor> gate,
+                             torch::Tensor k_cache, torch::Tensor v_cache,
+                             torch::Tensor block_table,
+                             torch::Tensor seq_lens, double scale,
+                             long window, long keep_first, bool sink);
 void mla_paged_attention(torch::Tensor out, torch::Tensor q,
                          torch::Tensor k_cache, torch::Tensor block_table,
                          torch::Tensor seq_lens,
@@ -115,6 +121,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "varlen MFMA paged prefill attention");
   m.def("window_attention_mfma", &window_attention_mfma,
         "prefill MFMA kernel with window + kept first tokens + sink + gate");
+  m.def("window_attention_decode", &window_attention_decode,
+        "split-KV decode kernels with window + kept first + sink + gate; "
+        "false = geometry not instantiated");
   m.def("skinny_gemm", &skinny_gemm,
         "decode-regime weight-streaming GEMM (M<=256)");
   m.def("mla_paged_attention", &mla_paged_attention,

@@ -32,6 +32,12 @@ void window_attention_mfma(torch::Tensor out, torch::Tensor q,
                            torch::Tensor query_start_loc, long max_query_len,
                            double scale, long window, long keep_first,
                            bool sink);
+bool window_attention_decode(torch::Tensor out, torch::Tensor q,
+                             c10::optional<torch::Tensor> gate,
+                             torch::Tensor k_cache, torch::Tensor v_cache,
+                             torch::Tensor block_table,
+                             torch::Tensor seq_lens, double scale,
+                             long window, long keep_first, bool sink);
 void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                       torch::Tensor conv_state, torch::Tensor slots,
                       torch::Tensor has_init, torch::Tensor query_start_loc);
@@ -65,6 +71,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "ragged paged attention: window + kept first tokens + sink + gate");
   m.def("window_attention_mfma", &window_attention_mfma,
         "MFMA tile form (bf16, D == Dv in {64,128}) of window_attention");
+  m.def("window_attention_decode", &window_attention_decode,
+        "split-KV decode kernels with window + kept first + sink + gate; "
+        "false = geometry not instantiated");
   m.def("causal_conv_silu", &causal_conv_silu,
         "ragged short causal conv + silu with per-slot state");
   m.def("delta_rule_varlen", &delta_rule_varlen,

@@ -92,9 +92,34 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(
   for (int i = 0; i < taps - 1; ++i) st[i] = next[i];
 }
 
+// One lane's contiguous key slice [i0, i0 + KP) of a q or k row as fp32;
+// 16 B vector loads when the host found every slice aligned and whole.
+template <typename T, int KP>
+DEV_INLINE void load_slice(const T *__restrict__ row, int i0, int Dk,
+                           bool vec, float *out) {
+  if (vec) {
+    if (sizeof(T) == 2) {
+#pragma unroll
+      for (int r = 0; r < KP; r += 8)
+        unpack8<T>(*reinterpret_cast<const shortx8 *>(row + i0 + r), out + r);
+    } else {
+#pragma unroll
+      for (int r = 0; r < KP; r += 4) {
+        const floatx4 f = *reinterpret_cast<const floatx4 *>(row + i0 + r);
+        out[r] = f[0]; out[r + 1] = f[1]; out[r + 2] = f[2]; out[r + 3] = f[3];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < KP; ++r)
+      out[r] = (i0 + r < Dk) ? ScalarOps<T>::to_f32(row[i0 + r]) : 0.f;
+  }
+}
+
 // grid (B, H, ceil(Dv / 64)), block 256 = 4 independent waves.
-// KP = key elements per lane = ceil(Dk / 4); lane (part, col) holds
-// S[part + 4 r][col] for r < KP.
+// KP = key elements per lane = ceil(Dk / 4) rounded up to 8/16/32/64;
+// lane (part, col) holds S[part * KP + r][col] for r < KP. The next
+// token's operands are loaded while the current one is computed.
 template <typename T, int KP>
 __global__ __launch_bounds__(256) void delta_rule_varlen_kernel(
     float *__restrict__ o, const T *__restrict__ q, const T *__restrict__ k,
@@ -103,42 +128,56 @@ __global__ __launch_bounds__(256) void delta_rule_varlen_kernel(
     const float *__restrict__ A_log, const float *__restrict__ dt_bias,
     float *__restrict__ state, const long *__restrict__ slots,
     const int *__restrict__ has_init, const int *__restrict__ qsl, int H,
-    int G, int Dk, int Dv, float q_scale) {
+    int G, int Dk, int Dv, float q_scale, int vec) {
   const int b = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = blockIdx.z * 64 + wave * 16 + (lane & 15);
   const int part = lane >> 4;
+  const int i0 = part * KP;
   const int g = h / (H / G);
   const int start = qsl[b], end = qsl[b + 1];
   const bool live = col < Dv;
   const int colc = live ? col : Dv - 1;  // clamp loads, mask stores
   if (blockIdx.z * 64 + wave * 16 >= Dv) return;  // whole wave idle
+  if (start >= end) return;
 
   float *sp = state + ((long)slots[b] * H + h) * Dk * Dv;
   float S[KP];
   const bool init = has_init[b] != 0;
 #pragma unroll
   for (int r = 0; r < KP; ++r) {
-    const int i = part + 4 * r;
+    const int i = i0 + r;
     S[r] = (init && i < Dk) ? sp[(long)i * Dv + colc] : 0.f;
   }
   const float neg_rate = -expf(A_log[h]);
   const float dtb = dt_bias[h];
 
+  float kc[KP], qc[KP];
+  float vc, ac, bc;
+  {
+    const long t = start;
+    load_slice<T, KP>(k + t * qkv_stride + (long)g * Dk, i0, Dk, vec, kc);
+    load_slice<T, KP>(q + t * qkv_stride + (long)g * Dk, i0, Dk, vec, qc);
+    vc = ScalarOps<T>::to_f32(v[t * qkv_stride + (long)h * Dv + colc]);
+    ac = ScalarOps<T>::to_f32(a[t * ab_stride + h]);
+    bc = ScalarOps<T>::to_f32(bproj[t * ab_stride + h]);
+  }
   for (int t = start; t < end; ++t) {
-    const T *qr = q + (long)t * qkv_stride + (long)g * Dk;
-    const T *kr = k + (long)t * qkv_stride + (long)g * Dk;
-    float kn[KP], qn[KP];
+    // prefetch t + 1 (clamped: the last iteration re-reads row t)
+    const long tn = t + 1 < end ? t + 1 : t;
+    float kx[KP], qx[KP];
+    load_slice<T, KP>(k + tn * qkv_stride + (long)g * Dk, i0, Dk, vec, kx);
+    load_slice<T, KP>(q + tn * qkv_stride + (long)g * Dk, i0, Dk, vec, qx);
+    const float vx =
+        ScalarOps<T>::to_f32(v[tn * qkv_stride + (long)h * Dv + colc]);
+    const float ax = ScalarOps<T>::to_f32(a[tn * ab_stride + h]);
+    const float bx = ScalarOps<T>::to_f32(bproj[tn * ab_stride + h]);
+
     float sk = 0.f, sq = 0.f;
 #pragma unroll
     for (int r = 0; r < KP; ++r) {
-      const int i = part + 4 * r;
-      const float kv = i < Dk ? ScalarOps<T>::to_f32(kr[i]) : 0.f;
-      const float qv = i < Dk ? ScalarOps<T>::to_f32(qr[i]) : 0.f;
-      kn[r] = kv;
-      qn[r] = qv;
-      sk += kv * kv;
-      sq += qv * qv;
+      sk += kc[r] * kc[r];
+      sq += qc[r] * qc[r];
     }
     sk += __shfl_xor(sk, 16, 64);
     sk += __shfl_xor(sk, 32, 64);
@@ -146,39 +185,42 @@ __global__ __launch_bounds__(256) void delta_rule_varlen_kernel(
     sq += __shfl_xor(sq, 32, 64);
     const float ik = 1.0f / sqrtf(sk + 1e-6f);
     const float iq = q_scale / sqrtf(sq + 1e-6f);
-    const float vv =
-        ScalarOps<T>::to_f32(v[(long)t * qkv_stride + (long)h * Dv + colc]);
-    const float av = ScalarOps<T>::to_f32(a[(long)t * ab_stride + h]) + dtb;
-    const float bv = ScalarOps<T>::to_f32(bproj[(long)t * ab_stride + h]);
+    const float av = ac + dtb;
     // softplus without overflow: max(x, 0) + log1p(exp(-|x|))
     const float sp_a = fmaxf(av, 0.f) + log1pf(expf(-fabsf(av)));
     const float gdec = expf(neg_rate * sp_a);
-    const float beta = 1.0f / (1.0f + expf(-bv));
+    const float beta = 1.0f / (1.0f + expf(-bc));
     float sk_dot = 0.f;
 #pragma unroll
     for (int r = 0; r < KP; ++r) {
-      kn[r] *= ik;
-      qn[r] *= iq;
+      kc[r] *= ik;
       S[r] *= gdec;
-      sk_dot += S[r] * kn[r];
+      sk_dot += S[r] * kc[r];
     }
     sk_dot += __shfl_xor(sk_dot, 16, 64);
     sk_dot += __shfl_xor(sk_dot, 32, 64);
-    const float u = beta * (vv - sk_dot);
+    const float u = beta * (vc - sk_dot);
     float od = 0.f;
 #pragma unroll
     for (int r = 0; r < KP; ++r) {
-      S[r] += kn[r] * u;
-      od += S[r] * qn[r];
+      S[r] += kc[r] * u;
+      od += S[r] * qc[r];
     }
+    od *= iq;
     od += __shfl_xor(od, 16, 64);
     od += __shfl_xor(od, 32, 64);
     if (live && part == 0) o[((long)t * H + h) * Dv + col] = od;
+#pragma unroll
+    for (int r = 0; r < KP; ++r) {
+      kc[r] = kx[r];
+      qc[r] = qx[r];
+    }
+    vc = vx; ac = ax; bc = bx;
   }
   if (live) {
 #pragma unroll
     for (int r = 0; r < KP; ++r) {
-      const int i = part + 4 * r;
+      const int i = i0 + r;
       if (i < Dk) sp[(long)i * Dv + col] = S[r];
     }
   }
@@ -290,6 +332,14 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
   TORCH_CHECK(Dk <= 256, "delta rule: key size <= 256");
   auto stream = at::cuda::getCurrentCUDAStream();
   const dim3 grid(B, H, (Dv + 63) / 64);
+  // 16 B vector loads of the per-lane key slices: every slice whole
+  // (Dk = 4 KP) and every row / head / slice offset 16 B aligned
+  const int kp = Dk <= 32 ? 8 : Dk <= 64 ? 16 : Dk <= 128 ? 32 : 64;
+  const size_t es = q.element_size();
+  const int vec =
+      (Dk == 4 * kp && (q.stride(0) * es) % 16 == 0 && (Dk * es) % 16 == 0 &&
+       reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0 &&
+       reinterpret_cast<uintptr_t>(k.data_ptr()) % 16 == 0) ? 1 : 0;
 #define RUN(TT, KPV)                                                         \
   hipLaunchKernelGGL((delta_rule_varlen_kernel<TT, KPV>), grid, dim3(256),   \
                      0, stream, o.data_ptr<float>(),                         \
@@ -300,7 +350,7 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                      dt_bias.data_ptr<float>(), state.data_ptr<float>(),     \
                      slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
                      query_start_loc.data_ptr<int>(), H, G, Dk, Dv,          \
-                     (float)q_scale)
+                     (float)q_scale, vec)
 #define RUN_KP(TT)                                                           \
   if (Dk <= 32) RUN(TT, 8);                                                  \
   else if (Dk <= 64) RUN(TT, 16);                                            \

@@ -25,11 +25,55 @@ DEV_INLINE float ln_block_sum(float v, float *red) {
   return block_reduce_sum<LN_BLOCK>(v, red);
 }
 
+// 8 consecutive elements <-> fp32 (16 B per bf16 load, 2 x 16 B per fp32)
+template <typename T> DEV_INLINE void ld8(const T *p, float *f) {
+  unpack8<T>(*reinterpret_cast<const shortx8 *>(p), f);
+}
+template <> DEV_INLINE void ld8<float>(const float *p, float *f) {
+  const floatx4 a = *reinterpret_cast<const floatx4 *>(p);
+  const floatx4 b = *reinterpret_cast<const floatx4 *>(p + 4);
+  f[0] = a[0]; f[1] = a[1]; f[2] = a[2]; f[3] = a[3];
+  f[4] = b[0]; f[5] = b[1]; f[6] = b[2]; f[7] = b[3];
+}
+template <typename T> DEV_INLINE void st8(T *p, const float *f) {
+  *reinterpret_cast<shortx8 *>(p) = pack8<T>(f);
+}
+template <> DEV_INLINE void st8<float>(float *p, const float *f) {
+  *reinterpret_cast<floatx4 *>(p) = floatx4{f[0], f[1], f[2], f[3]};
+  *reinterpret_cast<floatx4 *>(p + 4) = floatx4{f[4], f[5], f[6], f[7]};
+}
+
+// row <- src (vec: width % 8 == 0 and 16 B aligned rows)
+template <typename T>
+DEV_INLINE void row_load(float *row, const T *src, int width, bool vec) {
+  if (vec) {
+    for (int i = threadIdx.x * 8; i < width; i += LN_BLOCK * 8)
+      ld8<T>(src + i, row + i);
+  } else {
+    for (int i = threadIdx.x; i < width; i += LN_BLOCK)
+      row[i] = ScalarOps<T>::to_f32(src[i]);
+  }
+}
+
+template <typename T>
+DEV_INLINE void row_store(T *dst, const float *row, int width, bool vec) {
+  if (vec) {
+    for (int i = threadIdx.x * 8; i < width; i += LN_BLOCK * 8)
+      st8<T>(dst + i, row + i);
+  } else {
+    for (int i = threadIdx.x; i < width; i += LN_BLOCK)
+      dst[i] = ScalarOps<T>::from_f32(row[i]);
+  }
+}
+
 // normalize the LDS row in place: row = (row - mean) / sqrt(var + eps) * w + b
+// Callers put a barrier between filling the row and this call (the
+// reductions walk the row with another thread-to-element mapping than
+// the 8-wide loads); the trailing barrier publishes the result.
 template <typename T>
 DEV_INLINE void ln_row(float *row, const T *__restrict__ w,
                        const T *__restrict__ b, float eps, int width,
-                       float *red) {
+                       float *red, bool vec) {
   float s = 0.f;
   for (int i = threadIdx.x; i < width; i += LN_BLOCK) s += row[i];
   const float mean = ln_block_sum(s, red) / width;
@@ -40,23 +84,35 @@ DEV_INLINE void ln_row(float *row, const T *__restrict__ w,
   }
   const float var = ln_block_sum(ss, red) / width;
   const float inv = 1.0f / sqrtf(var + eps);
-  for (int i = threadIdx.x; i < width; i += LN_BLOCK)
-    row[i] = (row[i] - mean) * inv * ScalarOps<T>::to_f32(w[i]) +
-             ScalarOps<T>::to_f32(b[i]);
+  if (vec) {
+    for (int i = threadIdx.x * 8; i < width; i += LN_BLOCK * 8) {
+      float wf[8], bf[8];
+      ld8<T>(w + i, wf);
+      ld8<T>(b + i, bf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        row[i + e] = (row[i + e] - mean) * inv * wf[e] + bf[e];
+    }
+  } else {
+    for (int i = threadIdx.x; i < width; i += LN_BLOCK)
+      row[i] = (row[i] - mean) * inv * ScalarOps<T>::to_f32(w[i]) +
+               ScalarOps<T>::to_f32(b[i]);
+  }
+  __syncthreads();
 }
 
 template <typename T>
 __global__ __launch_bounds__(LN_BLOCK) void layernorm_f32_kernel(
     T *__restrict__ out, const float *__restrict__ x,
-    const T *__restrict__ w, const T *__restrict__ b, float eps, int width) {
+    const T *__restrict__ w, const T *__restrict__ b, float eps, int width,
+    int vec) {
   extern __shared__ float row[];
   __shared__ float red[LN_BLOCK / WAVE_SIZE];
   const long base = (long)blockIdx.x * width;
-  for (int i = threadIdx.x; i < width; i += LN_BLOCK) row[i] = x[base + i];
+  row_load<float>(row, x + base, width, vec);
   __syncthreads();
-  ln_row<T>(row, w, b, eps, width, red);
-  for (int i = threadIdx.x; i < width; i += LN_BLOCK)
-    out[base + i] = ScalarOps<T>::from_f32(row[i]);
+  ln_row<T>(row, w, b, eps, width, red, vec);
+  row_store<T>(out + base, row, width, vec);
 }
 
 // x += LN(y; w_post, b_post); optionally h = LN(x; w_pre, b_pre)
@@ -65,25 +121,39 @@ __global__ __launch_bounds__(LN_BLOCK) void residual_layernorm_kernel(
     float *__restrict__ x, const T *__restrict__ y, long y_stride,
     const T *__restrict__ w_post, const T *__restrict__ b_post,
     T *__restrict__ h, const T *__restrict__ w_pre,
-    const T *__restrict__ b_pre, float eps, int width) {
+    const T *__restrict__ b_pre, float eps, int width, int vec) {
   extern __shared__ float row[];
   __shared__ float red[LN_BLOCK / WAVE_SIZE];
   const long base = (long)blockIdx.x * width;
-  const T *yr = y + (long)blockIdx.x * y_stride;
-  for (int i = threadIdx.x; i < width; i += LN_BLOCK)
-    row[i] = ScalarOps<T>::to_f32(yr[i]);
+  row_load<T>(row, y + (long)blockIdx.x * y_stride, width, vec);
   __syncthreads();
-  ln_row<T>(row, w_post, b_post, eps, width, red);
-  for (int i = threadIdx.x; i < width; i += LN_BLOCK) {
-    const float r = x[base + i] + row[i];
-    x[base + i] = r;
-    row[i] = r;
+  ln_row<T>(row, w_post, b_post, eps, width, red, vec);
+  if (vec) {
+    for (int i = threadIdx.x * 8; i < width; i += LN_BLOCK * 8) {
+      float xf[8];
+      ld8<float>(x + base + i, xf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        xf[e] += row[i + e];
+        row[i + e] = xf[e];
+      }
+      st8<float>(x + base + i, xf);
+    }
+  } else {
+    for (int i = threadIdx.x; i < width; i += LN_BLOCK) {
+      const float r = x[base + i] + row[i];
+      x[base + i] = r;
+      row[i] = r;
+    }
   }
   if (h == nullptr) return;
   __syncthreads();
-  ln_row<T>(row, w_pre, b_pre, eps, width, red);
-  for (int i = threadIdx.x; i < width; i += LN_BLOCK)
-    h[base + i] = ScalarOps<T>::from_f32(row[i]);
+  ln_row<T>(row, w_pre, b_pre, eps, width, red, vec);
+  row_store<T>(h + base, row, width, vec);
+}
+
+bool aligned16(const void *p) {
+  return reinterpret_cast<uintptr_t>(p) % 16 == 0;
 }
 
 void check_vec(const torch::Tensor &t, int width, at::ScalarType st) {
@@ -103,12 +173,15 @@ void layernorm_f32(torch::Tensor out, torch::Tensor x, torch::Tensor w,
   TORCH_CHECK(width > 0 && width * 4 <= 64 * 1024);
   check_vec(w, width, out.scalar_type());
   check_vec(b, width, out.scalar_type());
+  const int vec = (width % 8 == 0 && aligned16(x.data_ptr()) &&
+                   aligned16(out.data_ptr()) && aligned16(w.data_ptr()) &&
+                   aligned16(b.data_ptr())) ? 1 : 0;
   auto stream = at::cuda::getCurrentCUDAStream();
 #define RUN(T)                                                             \
   hipLaunchKernelGGL((layernorm_f32_kernel<T>), dim3(rows), dim3(LN_BLOCK), \
                      width * sizeof(float), stream, (T *)out.data_ptr(),   \
                      x.data_ptr<float>(), (const T *)w.data_ptr(),         \
-                     (const T *)b.data_ptr(), (float)eps, width)
+                     (const T *)b.data_ptr(), (float)eps, width, vec)
   if (out.scalar_type() == at::kBFloat16) RUN(__hip_bfloat16);
   else if (out.scalar_type() == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "layernorm_f32: bf16 or fp32 output");
@@ -143,6 +216,11 @@ void residual_layernorm(torch::Tensor x, torch::Tensor y,
     wp = w_pre->data_ptr();
     bp = b_pre->data_ptr();
   }
+  const int vec =
+      (width % 8 == 0 && aligned16(x.data_ptr()) && aligned16(y.data_ptr()) &&
+       (y.stride(0) * y.element_size()) % 16 == 0 &&
+       aligned16(w_post.data_ptr()) && aligned16(b_post.data_ptr()) &&
+       aligned16(hp) && aligned16(wp) && aligned16(bp)) ? 1 : 0;
   auto stream = at::cuda::getCurrentCUDAStream();
 #define RUN(T)                                                              \
   hipLaunchKernelGGL((residual_layernorm_kernel<T>), dim3(rows),            \
@@ -150,7 +228,7 @@ void residual_layernorm(torch::Tensor x, torch::Tensor y,
                      x.data_ptr<float>(), (const T *)y.data_ptr(),          \
                      (long)y.stride(0), (const T *)w_post.data_ptr(),       \
                      (const T *)b_post.data_ptr(), (T *)hp, (const T *)wp,  \
-                     (const T *)bp, (float)eps, width)
+                     (const T *)bp, (float)eps, width, vec)
   if (st == at::kBFloat16) RUN(__hip_bfloat16);
   else if (st == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "residual_layernorm: bf16 or fp32 sublayer output");

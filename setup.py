@@ -10,7 +10,7 @@ repo snapshots without a site-packages install:
   (layer norm over an fp32 residual, windowed sink attention, varlen
   gated delta rule) plus the grouped MoE GEMM they are served with —
   the only native code a Sudevik-style model needs, so a fresh
-  checkout can serve one after compiling six files instead of
+  checkout can serve one after compiling seven files instead of
   fifteen.
 
 ``GLLM_EXT=seq`` (or ``core``) restricts the build to one module.
@@ -32,8 +32,8 @@ HIP_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
 CXX_FLAGS = ["-O3", "-std=c++17"]
 
 SEQ_SOURCES = ["bindings_seq.cpp", "layernorm.hip", "attention_window.hip",
-               "attention_prefill.hip", "delta_rule.hip", "moe.hip",
-               "elementwise.hip"]
+               "attention_prefill.hip", "attention_decode.hip",
+               "delta_rule.hip", "moe.hip", "elementwise.hip"]
 CORE_SOURCES = ["bindings.cpp", "norm.hip", "elementwise.hip",
                 "attention_decode.hip", "attention_prefill.hip",
                 "attention_mla.hip", "moe.hip", "fp8.hip", "gdn.hip",

@@ -431,7 +431,7 @@ def test_far_state_survives_long_decoding(device, dtype):
     other[0] = (other[0] + 1) % cfg["vocab"]
     a = oracle.forward(cfg, w, toks)[-1].numpy()
     b = oracle.forward(cfg, w, other)[-1].numpy()
-    assert rel_err(b.astype(np.float32), a) > 10 * TOL[dtype]
+    assert rel_err(b.astype(np.float32), a) > 0.05
 
 
 @pytest.mark.parametrize("device,dtype", DEVICES)
@@ -477,11 +477,11 @@ def test_greedy_generation_through_the_scheduler(device, dtype):
         for tok in o.token_ids:
             logits = oracle.forward(cfg, w, seq)[-1]
             top2 = torch.topk(logits, 2).values
-            if float(top2[0] - top2[1]) < margin:
-                break  # a near-tie proves nothing either way
-            assert tok == int(logits.argmax()), (len(seq), tok)
+            if float(top2[0] - top2[1]) >= margin:
+                # (a near-tie proves nothing either way: follow the engine)
+                assert tok == int(logits.argmax()), (len(seq), tok)
+                checked += 1
             seq.append(tok)
-            checked += 1
     assert checked >= 8
 
 
@@ -520,7 +520,7 @@ def test_window_attention_kernels_match_reference(D, Dv, dtype, window,
     from gllm_amd.ops import torch_ref
     tdt = getattr(torch, dtype)
     g = torch.Generator().manual_seed(D + Dv + window)
-    page, G, H = 16, 2, 6
+    page, G, H = 16, 2, 8
     geo = [(0, 200), (37, 1), (130, 77), (300, 1), (5, 2), (63, 129)]
     lens = [p + n for p, n in geo]
     npages = sum(-(-L // page) for L in lens) + 3
@@ -545,15 +545,23 @@ def test_window_attention_kernels_match_reference(D, Dv, dtype, window,
             want = torch_ref.window_attention(
                 q.float(), None if gt is None else gt.float(), kc.float(),
                 vc.float(), bt, sl, qsl, scale, window, keep, sink)
-            for mql in (200, 1):
-                # mql == 1 forces the generic kernel on the same batch
-                got = ops.window_attention(
-                    q.cuda(), None if gt is None else gt.cuda(), kc.cuda(),
-                    vc.cuda(), bt.cuda(), sl.cuda(), qsl.cuda(), scale,
-                    window, keep, sink, mql).float().cpu()
-                tol = 2e-2 if dtype == "bfloat16" else 2e-5
-                err = (got - want).abs().max().item()
-                assert err < tol, (use_gate, sink, mql, err)
+            got = ops.window_attention(
+                q.cuda(), None if gt is None else gt.cuda(), kc.cuda(),
+                vc.cuda(), bt.cuda(), sl.cuda(), qsl.cuda(), scale,
+                window, keep, sink, 200).float().cpu()
+            tol = 2e-2 if dtype == "bfloat16" else 2e-5
+            err = (got - want).abs().max().item()
+            assert err < tol, (use_gate, sink, err)
+            # decode-only batch: one new token per sequence (bf16 with
+            # an instantiated geometry takes the split-KV kernels)
+            last = qsl[1:].long() - 1
+            ar = torch.arange(len(geo) + 1, dtype=torch.int32)
+            got = ops.window_attention(
+                q[last].cuda(), None if gt is None else gt[last].cuda(),
+                kc.cuda(), vc.cuda(), bt.cuda(), sl.cuda(), ar.cuda(),
+                scale, window, keep, sink, 1).float().cpu()
+            err = (got - want[last]).abs().max().item()
+            assert err < tol, ("decode", use_gate, sink, err)
 
 
 @pytest.mark.gpu
