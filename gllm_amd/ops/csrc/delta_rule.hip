@@ -14,11 +14,12 @@
 //                        o = S^T q
 //                      with q, k unit-normalised per head (q also scaled),
 //                      beta = sigmoid(b), g = exp(-exp(A_log) softplus(a + dt)).
-//                      A wavefront owns 16 state columns; its 64 lanes are
-//                      4 key-slices x 16 columns, reductions over the key
-//                      axis are two lane shuffles, and waves never meet at a
-//                      barrier: the state column block lives in registers
-//                      for the whole portion.
+//                      A wavefront owns 16 state columns; each column is
+//                      shared by a quad of lanes that split the key axis,
+//                      so reductions over it are two DPP quad swaps, and
+//                      waves never meet at a barrier: the state column
+//                      block lives in registers for the whole portion.
+//                      Norms and gates come from a per-token pre-pass.
 //   rms_gate           o / rms(o) * w * silu(z) per head
 //
 // State layouts: conv [slots, C, taps-1] (oldest first), recurrent
@@ -116,23 +117,74 @@ DEV_INLINE void load_slice(const T *__restrict__ row, int i0, int Dk,
   }
 }
 
+// Per-token scalars of the recurrence, computed once instead of by every
+// wave that needs them: prep[t] = [ik(G) | iq(G) | decay(H) | beta(H)]
+// with ik = 1/sqrt(|k|^2 + 1e-6), iq = q_scale/sqrt(|q|^2 + 1e-6),
+// decay = exp(-exp(A_log) softplus(a + dt_bias)), beta = sigmoid(b).
+// grid (tokens), block 64.
+template <typename T>
+__global__ __launch_bounds__(64) void delta_prep_kernel(
+    float *__restrict__ prep, const T *__restrict__ q,
+    const T *__restrict__ k, long qkv_stride, const T *__restrict__ a,
+    const T *__restrict__ bproj, long ab_stride,
+    const float *__restrict__ A_log, const float *__restrict__ dt_bias,
+    int H, int G, int Dk, float q_scale) {
+  const long t = blockIdx.x;
+  const int lane = threadIdx.x;
+  float *out = prep + t * (2 * G + 2 * H);
+  for (int g = 0; g < G; ++g) {
+    float sk = 0.f, sq = 0.f;
+    for (int i = lane; i < Dk; i += 64) {
+      const float kv = ScalarOps<T>::to_f32(k[t * qkv_stride + (long)g * Dk + i]);
+      const float qv = ScalarOps<T>::to_f32(q[t * qkv_stride + (long)g * Dk + i]);
+      sk += kv * kv;
+      sq += qv * qv;
+    }
+    sk = wave_reduce_sum(sk);
+    sq = wave_reduce_sum(sq);
+    if (lane == 0) {
+      out[g] = 1.0f / sqrtf(sk + 1e-6f);
+      out[G + g] = q_scale / sqrtf(sq + 1e-6f);
+    }
+  }
+  for (int h = lane; h < H; h += 64) {
+    const float av = ScalarOps<T>::to_f32(a[t * ab_stride + h]) + dt_bias[h];
+    const float bv = ScalarOps<T>::to_f32(bproj[t * ab_stride + h]);
+    // softplus without overflow: max(x, 0) + log1p(exp(-|x|))
+    const float sp_a = fmaxf(av, 0.f) + log1pf(expf(-fabsf(av)));
+    out[2 * G + h] = expf(-expf(A_log[h]) * sp_a);
+    out[2 * G + H + h] = 1.0f / (1.0f + expf(-bv));
+  }
+}
+
+// sum over the 4 adjacent lanes of a quad (DPP quad_perm: no LDS trip)
+DEV_INLINE float quad_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));  // [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+      0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));  // [2,3,0,1]
+  return v;
+}
+
 // grid (B, H, ceil(Dv / 64)), block 256 = 4 independent waves.
-// KP = key elements per lane = ceil(Dk / 4) rounded up to 8/16/32/64;
-// lane (part, col) holds S[part * KP + r][col] for r < KP. The next
-// token's operands are loaded while the current one is computed.
+// A wave owns 16 state columns; a quad of adjacent lanes shares a column
+// and splits the key axis in 4 contiguous slices of KP = ceil(Dk / 4)
+// (rounded up to 8/16/32/64): lane (col, part) holds S[part * KP + r][col].
+// With S' = g S the step is
+//   d = ik g (S^T k);  u = beta (v - d);  S <- g S + k (u ik);  o = iq S^T q
+// on raw (un-normalised) q, k; the next token's operands are loaded
+// while the current one is computed.
 template <typename T, int KP>
 __global__ __launch_bounds__(256) void delta_rule_varlen_kernel(
     float *__restrict__ o, const T *__restrict__ q, const T *__restrict__ k,
-    const T *__restrict__ v, long qkv_stride, const T *__restrict__ a,
-    const T *__restrict__ bproj, long ab_stride,
-    const float *__restrict__ A_log, const float *__restrict__ dt_bias,
+    const T *__restrict__ v, long qkv_stride, const float *__restrict__ prep,
     float *__restrict__ state, const long *__restrict__ slots,
     const int *__restrict__ has_init, const int *__restrict__ qsl, int H,
-    int G, int Dk, int Dv, float q_scale, int vec) {
+    int G, int Dk, int Dv, int vec) {
   const int b = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int col = blockIdx.z * 64 + wave * 16 + (lane & 15);
-  const int part = lane >> 4;
+  const int col = blockIdx.z * 64 + wave * 16 + (lane >> 2);
+  const int part = lane & 3;
   const int i0 = part * KP;
   const int g = h / (H / G);
   const int start = qsl[b], end = qsl[b + 1];
@@ -140,6 +192,7 @@ __global__ __launch_bounds__(256) void delta_rule_varlen_kernel(
   const int colc = live ? col : Dv - 1;  // clamp loads, mask stores
   if (blockIdx.z * 64 + wave * 16 >= Dv) return;  // whole wave idle
   if (start >= end) return;
+  const int PW = 2 * G + 2 * H;
 
   float *sp = state + ((long)slots[b] * H + h) * Dk * Dv;
   float S[KP];
@@ -149,18 +202,16 @@ __global__ __launch_bounds__(256) void delta_rule_varlen_kernel(
     const int i = i0 + r;
     S[r] = (init && i < Dk) ? sp[(long)i * Dv + colc] : 0.f;
   }
-  const float neg_rate = -expf(A_log[h]);
-  const float dtb = dt_bias[h];
 
   float kc[KP], qc[KP];
-  float vc, ac, bc;
+  float vc, ikc, iqc, gc, bc;
   {
     const long t = start;
     load_slice<T, KP>(k + t * qkv_stride + (long)g * Dk, i0, Dk, vec, kc);
     load_slice<T, KP>(q + t * qkv_stride + (long)g * Dk, i0, Dk, vec, qc);
     vc = ScalarOps<T>::to_f32(v[t * qkv_stride + (long)h * Dv + colc]);
-    ac = ScalarOps<T>::to_f32(a[t * ab_stride + h]);
-    bc = ScalarOps<T>::to_f32(bproj[t * ab_stride + h]);
+    const float *pp = prep + t * PW;
+    ikc = pp[g]; iqc = pp[G + g]; gc = pp[2 * G + h]; bc = pp[2 * G + H + h];
   }
   for (int t = start; t < end; ++t) {
     // prefetch t + 1 (clamped: the last iteration re-reads row t)
@@ -170,52 +221,40 @@ __global__ __launch_bounds__(256) void delta_rule_varlen_kernel(
     load_slice<T, KP>(q + tn * qkv_stride + (long)g * Dk, i0, Dk, vec, qx);
     const float vx =
         ScalarOps<T>::to_f32(v[tn * qkv_stride + (long)h * Dv + colc]);
-    const float ax = ScalarOps<T>::to_f32(a[tn * ab_stride + h]);
-    const float bx = ScalarOps<T>::to_f32(bproj[tn * ab_stride + h]);
+    const float *pn = prep + tn * PW;
+    const float ikx = pn[g], iqx = pn[G + g], gx = pn[2 * G + h],
+                bx = pn[2 * G + H + h];
 
-    float sk = 0.f, sq = 0.f;
+    float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;  // 4 chains, not one
 #pragma unroll
-    for (int r = 0; r < KP; ++r) {
-      sk += kc[r] * kc[r];
-      sq += qc[r] * qc[r];
+    for (int r = 0; r < KP; r += 4) {
+      d0 += S[r] * kc[r];
+      d1 += S[r + 1] * kc[r + 1];
+      d2 += S[r + 2] * kc[r + 2];
+      d3 += S[r + 3] * kc[r + 3];
     }
-    sk += __shfl_xor(sk, 16, 64);
-    sk += __shfl_xor(sk, 32, 64);
-    sq += __shfl_xor(sq, 16, 64);
-    sq += __shfl_xor(sq, 32, 64);
-    const float ik = 1.0f / sqrtf(sk + 1e-6f);
-    const float iq = q_scale / sqrtf(sq + 1e-6f);
-    const float av = ac + dtb;
-    // softplus without overflow: max(x, 0) + log1p(exp(-|x|))
-    const float sp_a = fmaxf(av, 0.f) + log1pf(expf(-fabsf(av)));
-    const float gdec = expf(neg_rate * sp_a);
-    const float beta = 1.0f / (1.0f + expf(-bc));
-    float sk_dot = 0.f;
+    const float sk_dot = quad_sum((d0 + d1) + (d2 + d3)) * (ikc * gc);
+    const float c = bc * (vc - sk_dot) * ikc;
+    float e0 = 0.f, e1 = 0.f, e2 = 0.f, e3 = 0.f;
 #pragma unroll
-    for (int r = 0; r < KP; ++r) {
-      kc[r] *= ik;
-      S[r] *= gdec;
-      sk_dot += S[r] * kc[r];
+    for (int r = 0; r < KP; r += 4) {
+      S[r] = S[r] * gc + kc[r] * c;
+      S[r + 1] = S[r + 1] * gc + kc[r + 1] * c;
+      S[r + 2] = S[r + 2] * gc + kc[r + 2] * c;
+      S[r + 3] = S[r + 3] * gc + kc[r + 3] * c;
+      e0 += S[r] * qc[r];
+      e1 += S[r + 1] * qc[r + 1];
+      e2 += S[r + 2] * qc[r + 2];
+      e3 += S[r + 3] * qc[r + 3];
     }
-    sk_dot += __shfl_xor(sk_dot, 16, 64);
-    sk_dot += __shfl_xor(sk_dot, 32, 64);
-    const float u = beta * (vc - sk_dot);
-    float od = 0.f;
-#pragma unroll
-    for (int r = 0; r < KP; ++r) {
-      S[r] += kc[r] * u;
-      od += S[r] * qc[r];
-    }
-    od *= iq;
-    od += __shfl_xor(od, 16, 64);
-    od += __shfl_xor(od, 32, 64);
+    const float od = quad_sum((e0 + e1) + (e2 + e3)) * iqc;
     if (live && part == 0) o[((long)t * H + h) * Dv + col] = od;
 #pragma unroll
     for (int r = 0; r < KP; ++r) {
       kc[r] = kx[r];
       qc[r] = qx[r];
     }
-    vc = vx; ac = ax; bc = bx;
+    vc = vx; ikc = ikx; iqc = iqx; gc = gx; bc = bx;
   }
   if (live) {
 #pragma unroll
@@ -340,17 +379,28 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
       (Dk == 4 * kp && (q.stride(0) * es) % 16 == 0 && (Dk * es) % 16 == 0 &&
        reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0 &&
        reinterpret_cast<uintptr_t>(k.data_ptr()) % 16 == 0) ? 1 : 0;
+  // per-token scalars first: [ik(G) | iq(G) | decay(H) | beta(H)]
+  auto prep = torch::empty({T, 2 * G + 2 * H},
+                           o.options().dtype(at::kFloat));
+#define PREP(TT)                                                             \
+  hipLaunchKernelGGL((delta_prep_kernel<TT>), dim3(T), dim3(64), 0, stream,  \
+                     prep.data_ptr<float>(), (const TT *)q.data_ptr(),       \
+                     (const TT *)k.data_ptr(), (long)q.stride(0),            \
+                     (const TT *)a.data_ptr(), (const TT *)b.data_ptr(),     \
+                     (long)a.stride(0), A_log.data_ptr<float>(),             \
+                     dt_bias.data_ptr<float>(), H, G, Dk, (float)q_scale)
+  if (st == at::kBFloat16) PREP(__hip_bfloat16);
+  else if (st == at::kFloat) PREP(float);
+  else TORCH_CHECK(false, "delta_rule_varlen: bf16 or fp32");
+#undef PREP
 #define RUN(TT, KPV)                                                         \
   hipLaunchKernelGGL((delta_rule_varlen_kernel<TT, KPV>), grid, dim3(256),   \
                      0, stream, o.data_ptr<float>(),                         \
                      (const TT *)q.data_ptr(), (const TT *)k.data_ptr(),     \
                      (const TT *)v.data_ptr(), (long)q.stride(0),            \
-                     (const TT *)a.data_ptr(), (const TT *)b.data_ptr(),     \
-                     (long)a.stride(0), A_log.data_ptr<float>(),             \
-                     dt_bias.data_ptr<float>(), state.data_ptr<float>(),     \
+                     prep.data_ptr<float>(), state.data_ptr<float>(),        \
                      slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
-                     query_start_loc.data_ptr<int>(), H, G, Dk, Dv,          \
-                     (float)q_scale, vec)
+                     query_start_loc.data_ptr<int>(), H, G, Dk, Dv, vec)
 #define RUN_KP(TT)                                                           \
   if (Dk <= 32) RUN(TT, 8);                                                  \
   else if (Dk <= 64) RUN(TT, 16);                                            \

@@ -152,6 +152,95 @@ __global__ __launch_bounds__(LN_BLOCK) void residual_layernorm_kernel(
   row_store<T>(h + base, row, width, vec);
 }
 
+// Wave-per-row form of residual_layernorm for 8-aligned widths up to
+// 512 * NCH: the row stays in registers (NCH chunks of 8 per lane), the
+// four statistics are wave reductions, and there is no LDS traffic or
+// barrier at all. 4 rows per workgroup.
+template <typename T, int NCH>
+__global__ __launch_bounds__(LN_BLOCK) void residual_layernorm_wave_kernel(
+    float *__restrict__ x, const T *__restrict__ y, long y_stride,
+    const T *__restrict__ w_post, const T *__restrict__ b_post,
+    T *__restrict__ h, const T *__restrict__ w_pre,
+    const T *__restrict__ b_pre, float eps, int width, long rows) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * (LN_BLOCK / 64) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const long base = row * width;
+  const T *yr = y + row * y_stride;
+  float r[NCH][8];
+  float s = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int i = (c * 64 + lane) * 8;
+    if (i < width) {
+      ld8<T>(yr + i, r[c]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r[c][e] = 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += r[c][e];
+  }
+  float mean = wave_reduce_sum(s) / width;
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    if ((c * 64 + lane) * 8 < width) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = r[c][e] - mean;
+        ss += d * d;
+      }
+    }
+  }
+  float inv = 1.0f / sqrtf(wave_reduce_sum(ss) / width + eps);
+  s = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int i = (c * 64 + lane) * 8;
+    if (i < width) {
+      float wf[8], bf[8], xf[8];
+      ld8<T>(w_post + i, wf);
+      ld8<T>(b_post + i, bf);
+      ld8<float>(x + base + i, xf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        xf[e] += (r[c][e] - mean) * inv * wf[e] + bf[e];
+        r[c][e] = xf[e];
+        s += xf[e];
+      }
+      st8<float>(x + base + i, xf);
+    }
+  }
+  if (h == nullptr) return;
+  mean = wave_reduce_sum(s) / width;
+  ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    if ((c * 64 + lane) * 8 < width) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = r[c][e] - mean;
+        ss += d * d;
+      }
+    }
+  }
+  inv = 1.0f / sqrtf(wave_reduce_sum(ss) / width + eps);
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int i = (c * 64 + lane) * 8;
+    if (i < width) {
+      float wf[8], bf[8], of[8];
+      ld8<T>(w_pre + i, wf);
+      ld8<T>(b_pre + i, bf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        of[e] = (r[c][e] - mean) * inv * wf[e] + bf[e];
+      st8<T>(h + base + i, of);
+    }
+  }
+}
+
 bool aligned16(const void *p) {
   return reinterpret_cast<uintptr_t>(p) % 16 == 0;
 }
@@ -222,6 +311,33 @@ void residual_layernorm(torch::Tensor x, torch::Tensor y,
        aligned16(w_post.data_ptr()) && aligned16(b_post.data_ptr()) &&
        aligned16(hp) && aligned16(wp) && aligned16(bp)) ? 1 : 0;
   auto stream = at::cuda::getCurrentCUDAStream();
+  if (vec && width <= 8192) {
+    const int nch = width <= 512 ? 1 : width <= 1024 ? 2 : width <= 2048 ? 4
+                    : width <= 4096 ? 8 : 16;
+    const long blocks = (rows + LN_BLOCK / 64 - 1) / (LN_BLOCK / 64);
+#define RUNW(T, N)                                                          \
+  hipLaunchKernelGGL((residual_layernorm_wave_kernel<T, N>), dim3(blocks),  \
+                     dim3(LN_BLOCK), 0, stream, x.data_ptr<float>(),        \
+                     (const T *)y.data_ptr(), (long)y.stride(0),            \
+                     (const T *)w_post.data_ptr(),                          \
+                     (const T *)b_post.data_ptr(), (T *)hp, (const T *)wp,  \
+                     (const T *)bp, (float)eps, width, rows)
+#define RUNW_N(T)                                                           \
+  switch (nch) {                                                            \
+    case 1: RUNW(T, 1); break;                                              \
+    case 2: RUNW(T, 2); break;                                              \
+    case 4: RUNW(T, 4); break;                                              \
+    case 8: RUNW(T, 8); break;                                              \
+    default: RUNW(T, 16); break;                                            \
+  }
+    if (st == at::kBFloat16) { RUNW_N(__hip_bfloat16) }
+    else if (st == at::kFloat) { RUNW_N(float) }
+    else TORCH_CHECK(false, "residual_layernorm: bf16 or fp32");
+#undef RUNW_N
+#undef RUNW
+    HIP_CHECK_KERNEL();
+    return;
+  }
 #define RUN(T)                                                              \
   hipLaunchKernelGGL((residual_layernorm_kernel<T>), dim3(rows),            \
                      dim3(LN_BLOCK), width * sizeof(float), stream,         \

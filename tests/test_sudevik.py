@@ -618,3 +618,34 @@ def test_delta_rule_kernels_match_reference(H, G, Dk, Dv, taps, dtype):
         assert (a - b).abs().max().item() < tol * scale, name
     # untouched slots stay as they were
     assert torch.equal(got[4][2], st[2]) and torch.equal(got[4][6], st[6])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width", [20, 32, 1000, 2048, 8200])
+def test_layernorm_kernels_match_reference(width, dtype):
+    """layernorm_f32 / residual_layernorm on the GPU (scalar, 8-wide LDS
+    and wave-per-row variants by width) against the torch reference."""
+    from gllm_amd import ops
+    from gllm_amd.ops import torch_ref
+    tdt = getattr(torch, dtype)
+    g = torch.Generator().manual_seed(width)
+    rows = 37
+    x = torch.randn(rows, width, generator=g) * 3
+    y = torch.randn(rows, width + 8, generator=g).to(tdt)[:, :width]
+    w1, b1, w2, b2 = [(torch.randn(width, generator=g) * 0.3 + s).to(tdt)
+                      for s in (1, 0, 1, 0)]
+    tol = 3e-2 if dtype == "bfloat16" else 1e-5
+    want = torch_ref.layernorm_f32(x, w1, b1, 1e-5, tdt).float()
+    got = ops.layernorm_f32(x.cuda(), w1.cuda(), b1.cuda(), 1e-5,
+                            tdt).float().cpu()
+    assert (got - want).abs().max() < tol
+    for pre in (None, (w2, b2)):
+        xc, xg = x.clone(), x.clone().cuda()
+        hw = torch_ref.residual_layernorm(xc, y, w1, b1, 1e-5, pre)
+        hg = ops.residual_layernorm(
+            xg, y.cuda(), w1.cuda(), b1.cuda(), 1e-5,
+            None if pre is None else (w2.cuda(), b2.cuda()))
+        assert (xg.cpu() - xc).abs().max() < 1e-5 * 10
+        if pre is not None:
+            assert (hg.float().cpu() - hw.float()).abs().max() < tol
