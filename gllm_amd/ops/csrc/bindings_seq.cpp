@@ -49,7 +49,11 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                        double q_scale);
 void rms_gate(torch::Tensor out, torch::Tensor o, torch::Tensor z,
               torch::Tensor w, long H, double eps);
-// shared with the full extension (moe.hip, elementwise.hip)
+// shared with the full extension (skinny_gemm.hip, moe.hip,
+// elementwise.hip): what ops.linear / FusedMoE dispatch to in bf16
+void skinny_gemm(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                 c10::optional<torch::Tensor> bias,
+                 torch::Tensor workspace, long splitk);
 void silu_and_mul(torch::Tensor out, torch::Tensor x);
 void moe_align(torch::Tensor topk_ids, long E_local, long expert_start,
                long block_m, torch::Tensor sorted_ids,
@@ -79,6 +83,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("delta_rule_varlen", &delta_rule_varlen,
         "ragged gated delta rule, fp32 state in registers");
   m.def("rms_gate", &rms_gate, "o / rms(o) * w * silu(z) per head");
+  m.def("skinny_gemm", &skinny_gemm,
+        "decode-regime weight-streaming GEMM (M<=256)");
   m.def("silu_and_mul", &silu_and_mul, "silu(x[:d]) * x[d:]");
   m.def("moe_align", &moe_align, "device-side moe_align_block_size");
   m.def("moe_gemm", &moe_gemm, "grouped MFMA GEMM over sorted pairs");

@@ -8,9 +8,10 @@ repo snapshots without a site-packages install:
 * ``gllm_amd._kernels``      every kernel family of the framework
 * ``gllm_amd._kernels_seq``  the dtype-generic sequence-mixer kernels
   (layer norm over an fp32 residual, windowed sink attention, varlen
-  gated delta rule) plus the grouped MoE GEMM they are served with —
+  gated delta rule) plus the grouped MoE GEMM, gated activations and
+  skinny GEMM that the linear / MoE layers dispatch to —
   the only native code a Sudevik-style model needs, so a fresh
-  checkout can serve one after compiling seven files instead of
+  checkout can serve one after compiling eight files instead of
   fifteen.
 
 ``GLLM_EXT=seq`` (or ``core``) restricts the build to one module.
@@ -33,7 +34,8 @@ CXX_FLAGS = ["-O3", "-std=c++17"]
 
 SEQ_SOURCES = ["bindings_seq.cpp", "layernorm.hip", "attention_window.hip",
                "attention_prefill.hip", "attention_decode.hip",
-               "delta_rule.hip", "moe.hip", "elementwise.hip"]
+               "delta_rule.hip", "moe.hip", "elementwise.hip",
+               "skinny_gemm.hip"]
 CORE_SOURCES = ["bindings.cpp", "norm.hip", "elementwise.hip",
                 "attention_decode.hip", "attention_prefill.hip",
                 "attention_mla.hip", "moe.hip", "fp8.hip", "gdn.hip",
