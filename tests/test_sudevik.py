@@ -508,8 +508,10 @@ def test_config_and_registry():
 @pytest.mark.gpu
 @pytest.mark.parametrize("D,Dv,dtype", [
     (64, 64, "bfloat16"), (128, 128, "bfloat16"), (64, 64, "float32"),
-    (24, 40, "bfloat16"), (16, 8, "float32"), (128, 64, "bfloat16")])
-@pytest.mark.parametrize("window,keep", [(50, 3), (0, 0), (130, 70)])
+    (24, 40, "bfloat16"), (16, 8, "float32"), (128, 64, "bfloat16"),
+    (32, 320, "float32"), (7, 3, "float32")])
+@pytest.mark.parametrize("window,keep", [(50, 3), (0, 0), (130, 70),
+                                         (10, 40)])
 def test_window_attention_kernels_match_reference(D, Dv, dtype, window,
                                                   keep):
     """Both GPU kernels (MFMA tiles for bf16 D == Dv in {64, 128} when a
