@@ -145,6 +145,7 @@ class DeltaMixer(nn.Module):
         self.norm_weight = nn.Parameter(torch.ones(Dv, dtype=dtype),
                                         requires_grad=False)
         self.out_proj = RowParallelLinear(H * Dv, width, params_dtype=dtype)
+        self._ones = None
 
     def shard_of(self, name: str) -> Optional[int]:
         order = ["q", "k", "v", "g", "a", "b"]
@@ -165,7 +166,18 @@ class DeltaMixer(nn.Module):
         a = proj[:, self.conv_dim + hv:self.conv_dim + hv + self.H]
         b = proj[:, self.conv_dim + hv + self.H:]
         pool = fctx.ssm_pool
-        slots, init = fctx.ssm_slots_t, fctx.ssm_has_init_t
+        if fctx.ssm_slots_dev is not None:
+            # captured decode bucket: persistent slot buffer, every row
+            # a one-token step on carried state (padding rows work on
+            # the pool's scratch slot)
+            slots = fctx.ssm_slots_dev[:T]
+            if self._ones is None or self._ones.numel() < T \
+                    or self._ones.device != h.device:
+                self._ones = torch.ones(max(T, 1024), dtype=torch.int32,
+                                        device=h.device)
+            init = self._ones[:T]
+        else:
+            slots, init = fctx.ssm_slots_t, fctx.ssm_has_init_t
         qsl = fctx.query_start_loc
         conv = ops.causal_conv_silu(
             mixed, self.conv_weight, pool.conv_state[self.ssm_layer_id],
@@ -220,9 +232,6 @@ class SudevikLayer(nn.Module):
 class SudevikForCausalLM(nn.Module):
     # ragged state kernels read slots / flags from device tensors
     wants_state_tensors = True
-    # decode capture is not wired for the ragged kernels' host-built
-    # per-step tensors; serve eagerly
-    supports_graph = False
 
     def __init__(self, cfg, engine_config):
         super().__init__()
@@ -284,6 +293,14 @@ class SudevikForCausalLM(nn.Module):
                                     layers=ssm_specs)
         self.final_norm = LayerNorm(width, eps, dtype)
         self.lm_head = ParallelLMHead(vocab, width, params_dtype=dtype)
+        # hipGraph decode buckets need a sync-free forward: bf16 with
+        # every MoE on the grouped GEMM (8-aligned width and ff); fp32
+        # and odd expert shapes take the host segment loop
+        self.supports_graph = dtype == torch.bfloat16 and all(
+            lay.mlp is None or (width % 8 == 0 and
+                                lay.mlp.experts.intermediate_per_rank % 8
+                                == 0)
+            for lay in mods)
 
     @property
     def num_local_layers(self):
