@@ -238,6 +238,14 @@ def hybrid_gdn_config(sz, vocab=32000):
             "vocab_size": vocab}
 
 
+# the same two 8-layer stacks as --model choices of the flagship workload
+# (scheduler policies, overlap engine, hipGraph decode buckets)
+MODELS["sudevik-w2048"] = ("Sudevik-w2048-8L",
+                           sudevik_config(COMPARE_SIZES["w2048"]))
+MODELS["hybrid-gdn-w2048"] = ("hybrid-GDN-w2048-8L",
+                              hybrid_gdn_config(COMPARE_SIZES["w2048"]))
+
+
 def mixer_compare(args):
     from gllm_amd.config import EngineConfig
     from gllm_amd.engine.llm import LLM

@@ -50,6 +50,25 @@ DEV_INLINE shortx8 pack8(const float *in) {
   return p;
 }
 
+// ---- 8 consecutive elements <-> fp32 (one 16 B access for 16-bit types,
+// two for fp32); pointers must be 16 B aligned ----
+template <typename T> DEV_INLINE void ld8(const T *p, float *f) {
+  unpack8<T>(*reinterpret_cast<const shortx8 *>(p), f);
+}
+template <> DEV_INLINE void ld8<float>(const float *p, float *f) {
+  const floatx4 a = *reinterpret_cast<const floatx4 *>(p);
+  const floatx4 b = *reinterpret_cast<const floatx4 *>(p + 4);
+  f[0] = a[0]; f[1] = a[1]; f[2] = a[2]; f[3] = a[3];
+  f[4] = b[0]; f[5] = b[1]; f[6] = b[2]; f[7] = b[3];
+}
+template <typename T> DEV_INLINE void st8(T *p, const float *f) {
+  *reinterpret_cast<shortx8 *>(p) = pack8<T>(f);
+}
+template <> DEV_INLINE void st8<float>(float *p, const float *f) {
+  *reinterpret_cast<floatx4 *>(p) = floatx4{f[0], f[1], f[2], f[3]};
+  *reinterpret_cast<floatx4 *>(p + 4) = floatx4{f[4], f[5], f[6], f[7]};
+}
+
 // ---- wave reductions (64-wide) ----
 DEV_INLINE float wave_reduce_sum(float v) {
 #pragma unroll

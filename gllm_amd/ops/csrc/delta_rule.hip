@@ -72,6 +72,48 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
   out[(long)t * C + c] = ScalarOps<T>::from_f32(silu_f(acc));
 }
 
+// 8 channels per thread, 16 B accesses (C % 8 == 0, aligned rows);
+// grid (tokens, ceil(C / 8 / 256)). The taps-1 first tokens of a portion
+// read their history from the per-slot state with scalar loads.
+template <typename T, int TAPS>
+__global__ __launch_bounds__(256) void causal_conv_silu8_kernel(
+    T *__restrict__ out, const T *__restrict__ x, long x_stride,
+    const T *__restrict__ w, const T *__restrict__ state,
+    const long *__restrict__ slots, const int *__restrict__ has_init,
+    const int *__restrict__ qsl, int B, int C) {
+  const int t = blockIdx.x;
+  const int c0 = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (c0 >= C) return;
+  const int b = find_seq(qsl, B, t);
+  const int start = qsl[b];
+  const int r = t - start;
+  float wf[8 * TAPS];  // [channel][tap], contiguous in memory
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) ld8<T>(w + (long)c0 * TAPS + j * 8, wf + j * 8);
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int tap = 0; tap < TAPS; ++tap) {
+    const int rel = r - (TAPS - 1 - tap);
+    float xv[8];
+    if (rel >= 0) {
+      ld8<T>(x + (long)(start + rel) * x_stride + c0, xv);
+    } else if (has_init[b] != 0) {
+      const T *st = state + ((long)slots[b] * C + c0) * (TAPS - 1);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        xv[e] = ScalarOps<T>::to_f32(st[e * (TAPS - 1) + TAPS - 1 + rel]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xv[e] = 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += xv[e] * wf[e * TAPS + tap];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = silu_f(acc[e]);
+  st8<T>(out + (long)t * C + c0, acc);
+}
+
 // grid (B, ceil(C / 256)); each thread owns one (sequence, channel) state
 template <typename T>
 __global__ __launch_bounds__(256) void conv_state_update_kernel(
@@ -286,6 +328,34 @@ __global__ __launch_bounds__(64) void rms_gate_kernel(
   }
 }
 
+// 8 elements per lane, LPR = Dv / 8 lanes per (token, head) row;
+// grid ceil(rows / (256 / LPR)), block 256
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void rms_gate8_kernel(
+    T *__restrict__ out, const float *__restrict__ o,
+    const T *__restrict__ z, long z_stride, const T *__restrict__ w,
+    int H, long rows, float eps) {
+  constexpr int Dv = LPR * 8;
+  const long th = (long)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
+  const int d0 = (threadIdx.x % LPR) * 8;
+  const bool ok = th < rows;
+  const long thc = ok ? th : rows - 1;  // whole groups take the reduction
+  const long t = thc / H;
+  const int h = thc % H;
+  float of[8], zf[8], wf[8];
+  ld8<float>(o + thc * Dv + d0, of);
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ss += of[e] * of[e];
+  ss = group_reduce_sum<LPR>(ss);
+  const float inv = 1.0f / sqrtf(ss / Dv + eps);
+  ld8<T>(z + t * z_stride + (long)h * Dv + d0, zf);
+  ld8<T>(w + d0, wf);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) of[e] = of[e] * inv * wf[e] * silu_f(zf[e]);
+  if (ok) st8<T>(out + th * Dv + d0, of);
+}
+
 bool rows_ok(const torch::Tensor &t) {
   return t.dim() == 2 && t.stride(1) == 1;
 }
@@ -314,14 +384,43 @@ void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
               query_start_loc.numel() >= B + 1);
   auto stream = at::cuda::getCurrentCUDAStream();
   const int cy = (C + 255) / 256;
-#define RUN(TT)                                                              \
-  hipLaunchKernelGGL((causal_conv_silu_kernel<TT>), dim3(T, cy), dim3(256),  \
-                     0, stream, (TT *)out.data_ptr(),                        \
+  const size_t es = x.element_size();
+  const bool vec8 =
+      C % 8 == 0 && (x.stride(0) * es) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(w.data_ptr()) % 16 == 0;
+  const int cy8 = (C / 8 + 255) / 256;
+#define CONV8(TT, TP)                                                        \
+  hipLaunchKernelGGL((causal_conv_silu8_kernel<TT, TP>), dim3(T, cy8),       \
+                     dim3(256), 0, stream, (TT *)out.data_ptr(),             \
                      (const TT *)x.data_ptr(), (long)x.stride(0),            \
                      (const TT *)w.data_ptr(),                               \
                      (const TT *)conv_state.data_ptr(),                      \
                      slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
-                     query_start_loc.data_ptr<int>(), B, C, taps);           \
+                     query_start_loc.data_ptr<int>(), B, C)
+#define CONV8_T(TT)                                                          \
+  switch (taps) {                                                            \
+    case 1: CONV8(TT, 1); break;                                             \
+    case 2: CONV8(TT, 2); break;                                             \
+    case 3: CONV8(TT, 3); break;                                             \
+    case 4: CONV8(TT, 4); break;                                             \
+    case 5: CONV8(TT, 5); break;                                             \
+    case 6: CONV8(TT, 6); break;                                             \
+    case 7: CONV8(TT, 7); break;                                             \
+    default: CONV8(TT, 8); break;                                            \
+  }
+#define RUN(TT)                                                              \
+  if (vec8) {                                                                \
+    CONV8_T(TT)                                                              \
+  } else                                                                     \
+    hipLaunchKernelGGL((causal_conv_silu_kernel<TT>), dim3(T, cy),           \
+                       dim3(256), 0, stream, (TT *)out.data_ptr(),           \
+                       (const TT *)x.data_ptr(), (long)x.stride(0),          \
+                       (const TT *)w.data_ptr(),                             \
+                       (const TT *)conv_state.data_ptr(),                    \
+                       slots.data_ptr<long>(), has_init.data_ptr<int>(),     \
+                       query_start_loc.data_ptr<int>(), B, C, taps);         \
   if (taps > 1)                                                              \
     hipLaunchKernelGGL((conv_state_update_kernel<TT>), dim3(B, cy),          \
                        dim3(256), 0, stream, (TT *)conv_state.data_ptr(),    \
@@ -332,6 +431,8 @@ void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
   else if (st == at::kFloat) { RUN(float); }
   else TORCH_CHECK(false, "causal_conv_silu: bf16 or fp32");
 #undef RUN
+#undef CONV8_T
+#undef CONV8
   HIP_CHECK_KERNEL();
 }
 
@@ -426,6 +527,39 @@ void rms_gate(torch::Tensor out, torch::Tensor o, torch::Tensor z,
               z.size(0) * H == rows);
   TORCH_CHECK(w.scalar_type() == st && w.is_contiguous());
   auto stream = at::cuda::getCurrentCUDAStream();
+  const int lpr = Dv / 8;
+  const bool vec8 =
+      Dv % 8 == 0 && lpr <= 64 && (lpr & (lpr - 1)) == 0 &&
+      (z.stride(0) * z.element_size()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(z.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(o.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(w.data_ptr()) % 16 == 0;
+  if (vec8) {
+    const long blocks = (rows * lpr + 255) / 256;
+#define G8(TT, L)                                                            \
+  hipLaunchKernelGGL((rms_gate8_kernel<TT, L>), dim3(blocks), dim3(256), 0,  \
+                     stream, (TT *)out.data_ptr(), o.data_ptr<float>(),      \
+                     (const TT *)z.data_ptr(), (long)z.stride(0),            \
+                     (const TT *)w.data_ptr(), (int)H, rows, (float)eps)
+#define G8_L(TT)                                                             \
+  switch (lpr) {                                                             \
+    case 1: G8(TT, 1); break;                                                \
+    case 2: G8(TT, 2); break;                                                \
+    case 4: G8(TT, 4); break;                                                \
+    case 8: G8(TT, 8); break;                                                \
+    case 16: G8(TT, 16); break;                                              \
+    case 32: G8(TT, 32); break;                                              \
+    default: G8(TT, 64); break;                                              \
+  }
+    if (st == at::kBFloat16) { G8_L(__hip_bfloat16) }
+    else if (st == at::kFloat) { G8_L(float) }
+    else TORCH_CHECK(false, "rms_gate: bf16 or fp32");
+#undef G8_L
+#undef G8
+    HIP_CHECK_KERNEL();
+    return;
+  }
 #define RUN(TT)                                                              \
   hipLaunchKernelGGL((rms_gate_kernel<TT>), dim3(rows), dim3(64), 0, stream, \
                      (TT *)out.data_ptr(), o.data_ptr<float>(),              \

@@ -25,24 +25,6 @@ DEV_INLINE float ln_block_sum(float v, float *red) {
   return block_reduce_sum<LN_BLOCK>(v, red);
 }
 
-// 8 consecutive elements <-> fp32 (16 B per bf16 load, 2 x 16 B per fp32)
-template <typename T> DEV_INLINE void ld8(const T *p, float *f) {
-  unpack8<T>(*reinterpret_cast<const shortx8 *>(p), f);
-}
-template <> DEV_INLINE void ld8<float>(const float *p, float *f) {
-  const floatx4 a = *reinterpret_cast<const floatx4 *>(p);
-  const floatx4 b = *reinterpret_cast<const floatx4 *>(p + 4);
-  f[0] = a[0]; f[1] = a[1]; f[2] = a[2]; f[3] = a[3];
-  f[4] = b[0]; f[5] = b[1]; f[6] = b[2]; f[7] = b[3];
-}
-template <typename T> DEV_INLINE void st8(T *p, const float *f) {
-  *reinterpret_cast<shortx8 *>(p) = pack8<T>(f);
-}
-template <> DEV_INLINE void st8<float>(float *p, const float *f) {
-  *reinterpret_cast<floatx4 *>(p) = floatx4{f[0], f[1], f[2], f[3]};
-  *reinterpret_cast<floatx4 *>(p + 4) = floatx4{f[4], f[5], f[6], f[7]};
-}
-
 // row <- src (vec: width % 8 == 0 and 16 B aligned rows)
 template <typename T>
 DEV_INLINE void row_load(float *row, const T *src, int width, bool vec) {

@@ -574,10 +574,11 @@ def test_window_attention_kernels_match_reference(D, Dv, dtype, window,
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("off", [3, 8], ids=["unaligned", "aligned"])
 @pytest.mark.parametrize("H,G,Dk,Dv,taps", [
     (4, 2, 128, 128, 4), (3, 1, 20, 5, 2), (2, 2, 64, 96, 3),
-    (8, 4, 32, 16, 1), (2, 1, 200, 72, 8)])
-def test_delta_rule_kernels_match_reference(H, G, Dk, Dv, taps, dtype):
+    (8, 4, 32, 16, 1), (2, 1, 200, 72, 8), (4, 4, 16, 64, 5)])
+def test_delta_rule_kernels_match_reference(H, G, Dk, Dv, taps, dtype, off):
     """causal_conv_silu + delta_rule_varlen + rms_gate on the GPU against
     the torch reference of the same ops: ragged batch (fresh portions,
     continued portions, decode tokens), state slots out of order."""
@@ -593,7 +594,9 @@ def test_delta_rule_kernels_match_reference(H, G, Dk, Dv, taps, dtype):
     qsl = torch.tensor([0] + list(np.cumsum([n for _, n in geo])),
                        dtype=torch.int32)
     init = torch.tensor([int(i) for i, _ in geo], dtype=torch.int32)
-    x = torch.randn(T, C + 7, generator=g).to(tdt)[:, 3:3 + C]  # a slice
+    # a column slice of a wider buffer; the aligned one takes the 16 B
+    # vector kernels where the shapes allow
+    x = torch.randn(T, C + 16, generator=g).to(tdt)[:, off:off + C]
     w = (torch.randn(C, taps, generator=g) * 0.5).to(tdt)
     cs = torch.randn(n_slots, C, max(taps - 1, 1), generator=g).to(tdt)
     st = torch.randn(n_slots, H, Dk, Dv, generator=g) * 0.3
