@@ -235,10 +235,13 @@ def tokens_for(cfg, n, seed):
     [with_moe(attn(), experts=3, top=3, ff=24)],
 ], ids=["delta", "delta-odd", "attn", "attn-plain", "attn-mqa", "attn-moe",
         "moe-all-experts"])
-def test_each_mechanism_alone(layers, device, dtype):
+@pytest.mark.parametrize("width", [32, 36], ids=["w32", "w36"])
+def test_each_mechanism_alone(layers, device, dtype, width):
     """One-layer models: each mixer / feed-forward on its own, every
-    position of a whole prompt (the first tokens included)."""
-    cfg = make_config(layers)
+    position of a whole prompt (the first tokens included). Width 36 is
+    not a multiple of 8: scalar norm kernels, unaligned projection rows,
+    experts on the segment loop."""
+    cfg = make_config(layers, width=width)
     w = make_weights(cfg, 1)
     llm = engine(save_model(cfg, w), device, dtype)
     toks = tokens_for(cfg, 37, 2)
