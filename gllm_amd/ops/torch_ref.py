@@ -301,13 +301,11 @@ def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
     q.copy_(prep(q, q_w, H).reshape(T, H * D).to(q.dtype))
     if k is None:
         return
-    page = k_cache.shape[1]
     rows = slot_mapping[:T]
     kc = k_cache.view(-1, G, D)
     vc = v_cache.view(-1, G, Dv)
     kc[rows] = prep(k, k_w, G).to(k_cache.dtype)
     vc[rows] = v.reshape(T, G, Dv).to(v_cache.dtype)
-    del page
 
 
 def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,

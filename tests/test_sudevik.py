@@ -9,7 +9,6 @@ ops; the same tests marked ``gpu`` exercise the HIP kernels in fp32
 (tight tolerance) and bf16.
 """
 
-import io
 import json
 import os
 import tempfile
