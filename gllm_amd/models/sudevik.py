@@ -185,7 +185,7 @@ class DeltaMixer(nn.Module):
         o = ops.delta_rule_varlen(
             conv[:, :gk], conv[:, gk:2 * gk], conv[:, 2 * gk:], a, b,
             self.A_log, self.dt_bias, pool.ssm_state[self.ssm_layer_id],
-            slots, init, qsl, self.Dk ** -0.5)
+            slots, init, qsl, self.Dk ** -0.5, fctx.max_query_len)
         gated = ops.rms_gate(o, z, self.norm_weight, self.H, self.eps,
                              h.dtype)
         return self.out_proj(gated)

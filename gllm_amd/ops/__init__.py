@@ -839,17 +839,21 @@ def causal_conv_silu(x, w, conv_state, slots, has_init, query_start_loc):
 
 
 def delta_rule_varlen(q, k, v, a, b, A_log, dt_bias, state, slots,
-                      has_init, query_start_loc, q_scale) -> torch.Tensor:
+                      has_init, query_start_loc, q_scale,
+                      max_query_len=0) -> torch.Tensor:
     """Ragged gated delta rule (prompt portions and decode tokens in one
     launch); fp32 state [slots, H, Dk, Dv] in place; returns fp32
-    [T, H, Dv]."""
+    [T, H, Dv]. ``max_query_len`` == 1 (decode-only batch) keeps the
+    operands in registers; anything else stages token tiles through
+    LDS — same arithmetic per token either way."""
     if q.is_cuda:
         H, _, Dv = state.shape[1:]
         o = torch.empty(q.shape[0], H, Dv, dtype=torch.float32,
                         device=q.device)
         _seq_kernels().delta_rule_varlen(o, q, k, v, a, b, A_log, dt_bias,
                                          state, slots, has_init,
-                                         query_start_loc, q_scale)
+                                         query_start_loc, q_scale,
+                                         max_query_len)
         return o
     from gllm_amd.ops import gdn_ref
     return gdn_ref.delta_rule_varlen(q, k, v, a, b, A_log, dt_bias, state,

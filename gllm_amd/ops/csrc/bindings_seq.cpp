@@ -46,7 +46,7 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                        torch::Tensor A_log, torch::Tensor dt_bias,
                        torch::Tensor state, torch::Tensor slots,
                        torch::Tensor has_init, torch::Tensor query_start_loc,
-                       double q_scale);
+                       double q_scale, long max_query_len);
 void rms_gate(torch::Tensor out, torch::Tensor o, torch::Tensor z,
               torch::Tensor w, long H, double eps);
 // shared with the full extension (skinny_gemm.hip, moe.hip,

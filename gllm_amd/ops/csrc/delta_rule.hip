@@ -307,6 +307,164 @@ __global__ __launch_bounds__(256) void delta_rule_varlen_kernel(
   }
 }
 
+// Prompt-portion form of the same recurrence: the 4 waves of a workgroup
+// share q, k (one kv head) and the per-token scalars, so tiles of TT
+// tokens are staged once per workgroup into LDS as fp32 (double buffered:
+// the next tile's global loads are in flight while the current one is
+// computed) and every lane reads its key slice with 16 B LDS loads. The
+// arithmetic per token is exactly delta_rule_varlen_kernel's.
+// grid (B, H, ceil(Dv / 64)), block 256.
+template <typename T, int KP>
+__global__ __launch_bounds__(256) void delta_rule_tiled_kernel(
+    float *__restrict__ o, const T *__restrict__ q, const T *__restrict__ k,
+    const T *__restrict__ v, long qkv_stride, const float *__restrict__ prep,
+    float *__restrict__ state, const long *__restrict__ slots,
+    const int *__restrict__ has_init, const int *__restrict__ qsl, int H,
+    int G, int Dk, int Dv) {
+  constexpr int TT = KP == 64 ? 8 : 16;   // tokens per tile
+  constexpr int KPP = KP + 4;             // padded slice: no bank clash
+  constexpr int DKP = 4 * KP;             // padded key size
+  constexpr int KQ_T = 2 * 4 * KPP;       // floats per token: [k|q][part]
+  constexpr int TOK_F = KQ_T + 64 + 4;    // + v columns + 4 scalars
+  constexpr int PER = TT * 2 * DKP / 256; // k/q elements per thread, tile
+  constexpr int VPER = TT * 64 / 256;
+  __shared__ __attribute__((aligned(16))) float lds[2][TT * TOK_F];
+
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int vcol = wave * 16 + (lane >> 2);  // column inside the 64 block
+  const int col = blockIdx.z * 64 + vcol;
+  const int part = lane & 3;
+  const int i0 = part * KP;
+  const int g = h / (H / G);
+  const int start = qsl[b], end = qsl[b + 1];
+  if (start >= end) return;
+  const bool live = col < Dv;
+  const int colc = live ? col : Dv - 1;
+  const int PW = 2 * G + 2 * H;
+
+  float *sp = state + ((long)slots[b] * H + h) * Dk * Dv;
+  float S[KP];
+  const bool init = has_init[b] != 0;
+#pragma unroll
+  for (int r = 0; r < KP; ++r) {
+    const int i = i0 + r;
+    S[r] = (init && i < Dk) ? sp[(long)i * Dv + colc] : 0.f;
+  }
+
+  T stg[PER];
+  T stg_v[VPER];
+  float stg_s = 0.f;
+  auto stage_load = [&](int tile0) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int idx = j * 256 + tid;
+      const int tt = idx / (2 * DKP);
+      const int w = (idx / DKP) & 1;
+      const int i = idx % DKP;
+      const long t = tile0 + tt;
+      const T *src = w ? q : k;
+      stg[j] = (i < Dk && t < end) ? src[t * qkv_stride + (long)g * Dk + i]
+                                   : ScalarOps<T>::from_f32(0.f);
+    }
+#pragma unroll
+    for (int j = 0; j < VPER; ++j) {
+      const int idx = j * 256 + tid;
+      const int tt = idx / 64, c = blockIdx.z * 64 + idx % 64;
+      const long t = tile0 + tt;
+      stg_v[j] = (c < Dv && t < end)
+                     ? v[t * qkv_stride + (long)h * Dv + c]
+                     : ScalarOps<T>::from_f32(0.f);
+    }
+    if (tid < TT * 4) {
+      const int tt = tid >> 2, which = tid & 3;
+      const long t = tile0 + tt < end ? tile0 + tt : end - 1;
+      const float *pp = prep + t * PW;
+      stg_s = which == 0 ? pp[g] : which == 1 ? pp[G + g]
+              : which == 2 ? pp[2 * G + h] : pp[2 * G + H + h];
+    }
+  };
+  auto stage_store = [&](float *buf) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int idx = j * 256 + tid;
+      const int tt = idx / (2 * DKP);
+      const int w = (idx / DKP) & 1;
+      const int i = idx % DKP;
+      buf[tt * TOK_F + (w * 4 + i / KP) * KPP + i % KP] =
+          ScalarOps<T>::to_f32(stg[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < VPER; ++j) {
+      const int idx = j * 256 + tid;
+      buf[(idx / 64) * TOK_F + KQ_T + idx % 64] =
+          ScalarOps<T>::to_f32(stg_v[j]);
+    }
+    if (tid < TT * 4) buf[(tid >> 2) * TOK_F + KQ_T + 64 + (tid & 3)] = stg_s;
+  };
+
+  stage_load(start);
+  stage_store(lds[0]);
+  __syncthreads();
+  int cur = 0;
+  for (int tile0 = start; tile0 < end; tile0 += TT) {
+    const bool more = tile0 + TT < end;
+    if (more) stage_load(tile0 + TT);
+    const int n = end - tile0 < TT ? end - tile0 : TT;
+    const float *buf = lds[cur];
+    for (int tt = 0; tt < n; ++tt) {
+      const float *tok = buf + tt * TOK_F;
+      const floatx4 *kp4 =
+          reinterpret_cast<const floatx4 *>(tok + part * KPP);
+      const floatx4 *qp4 =
+          reinterpret_cast<const floatx4 *>(tok + (4 + part) * KPP);
+      const float vc = tok[KQ_T + vcol];
+      const float ikc = tok[KQ_T + 64], iqc = tok[KQ_T + 65];
+      const float gc = tok[KQ_T + 66], bc = tok[KQ_T + 67];
+      float kc[KP];
+      float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+      for (int r = 0; r < KP; r += 4) {
+        const floatx4 kk = kp4[r / 4];
+        kc[r] = kk[0]; kc[r + 1] = kk[1]; kc[r + 2] = kk[2]; kc[r + 3] = kk[3];
+        d0 += S[r] * kk[0];
+        d1 += S[r + 1] * kk[1];
+        d2 += S[r + 2] * kk[2];
+        d3 += S[r + 3] * kk[3];
+      }
+      const float sk_dot = quad_sum((d0 + d1) + (d2 + d3)) * (ikc * gc);
+      const float c = bc * (vc - sk_dot) * ikc;
+      float e0 = 0.f, e1 = 0.f, e2 = 0.f, e3 = 0.f;
+#pragma unroll
+      for (int r = 0; r < KP; r += 4) {
+        const floatx4 qq = qp4[r / 4];
+        S[r] = S[r] * gc + kc[r] * c;
+        S[r + 1] = S[r + 1] * gc + kc[r + 1] * c;
+        S[r + 2] = S[r + 2] * gc + kc[r + 2] * c;
+        S[r + 3] = S[r + 3] * gc + kc[r + 3] * c;
+        e0 += S[r] * qq[0];
+        e1 += S[r + 1] * qq[1];
+        e2 += S[r + 2] * qq[2];
+        e3 += S[r + 3] * qq[3];
+      }
+      const float od = quad_sum((e0 + e1) + (e2 + e3)) * iqc;
+      if (live && part == 0)
+        o[((long)(tile0 + tt) * H + h) * Dv + col] = od;
+    }
+    if (more) stage_store(lds[cur ^ 1]);
+    __syncthreads();
+    cur ^= 1;
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < KP; ++r) {
+      const int i = i0 + r;
+      if (i < Dk) sp[(long)i * Dv + col] = S[r];
+    }
+  }
+}
+
 // grid (tokens * H); block 64: out = o / rms(o) * w * silu(z)
 template <typename T>
 __global__ __launch_bounds__(64) void rms_gate_kernel(
@@ -441,7 +599,7 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                        torch::Tensor A_log, torch::Tensor dt_bias,
                        torch::Tensor state, torch::Tensor slots,
                        torch::Tensor has_init, torch::Tensor query_start_loc,
-                       double q_scale) {
+                       double q_scale, long max_query_len) {
   const long T = q.size(0);
   if (T == 0) return;
   const auto st = q.scalar_type();
@@ -502,8 +660,24 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
                      prep.data_ptr<float>(), state.data_ptr<float>(),        \
                      slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
                      query_start_loc.data_ptr<int>(), H, G, Dk, Dv, vec)
+#define RUNT(TT, KPV)                                                        \
+  hipLaunchKernelGGL((delta_rule_tiled_kernel<TT, KPV>), grid, dim3(256),    \
+                     0, stream, o.data_ptr<float>(),                         \
+                     (const TT *)q.data_ptr(), (const TT *)k.data_ptr(),     \
+                     (const TT *)v.data_ptr(), (long)q.stride(0),            \
+                     prep.data_ptr<float>(), state.data_ptr<float>(),        \
+                     slots.data_ptr<long>(), has_init.data_ptr<int>(),       \
+                     query_start_loc.data_ptr<int>(), H, G, Dk, Dv)
+  // batches that hold a prompt portion stage tiles through LDS; decode-
+  // only batches (one token per sequence) keep everything in registers
+  const bool tiled = max_query_len != 1;
 #define RUN_KP(TT)                                                           \
-  if (Dk <= 32) RUN(TT, 8);                                                  \
+  if (tiled) {                                                               \
+    if (Dk <= 32) RUNT(TT, 8);                                               \
+    else if (Dk <= 64) RUNT(TT, 16);                                         \
+    else if (Dk <= 128) RUNT(TT, 32);                                        \
+    else RUNT(TT, 64);                                                       \
+  } else if (Dk <= 32) RUN(TT, 8);                                           \
   else if (Dk <= 64) RUN(TT, 16);                                            \
   else if (Dk <= 128) RUN(TT, 32);                                           \
   else RUN(TT, 64)
@@ -511,6 +685,7 @@ void delta_rule_varlen(torch::Tensor o, torch::Tensor q, torch::Tensor k,
   else if (st == at::kFloat) { RUN_KP(float); }
   else TORCH_CHECK(false, "delta_rule_varlen: bf16 or fp32");
 #undef RUN_KP
+#undef RUNT
 #undef RUN
   HIP_CHECK_KERNEL();
 }

@@ -5,7 +5,7 @@
 Two extension modules land next to the package so they travel with
 repo snapshots without a site-packages install:
 
-* ``gllm_amd._kernels``      every kernel family of the framework
+* ``gllm_amd._kernels``      the kernel families of the other models
 * ``gllm_amd._kernels_seq``  the dtype-generic sequence-mixer kernels
   (layer norm over an fp32 residual, windowed sink attention, varlen
   gated delta rule) plus the grouped MoE GEMM, gated activations and

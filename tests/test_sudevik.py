@@ -608,7 +608,7 @@ def test_delta_rule_kernels_match_reference(H, G, Dk, Dv, taps, dtype, off):
     z = torch.randn(T, H * Dv, generator=g).to(tdt)
     nw = (1 + 0.2 * torch.randn(Dv, generator=g)).to(tdt)
 
-    def run(dev):
+    def run(dev, mql=0):
         cs_d, st_d = cs.clone().to(dev), st.clone().to(dev)
         conv = ops.causal_conv_silu(x.to(dev), w.to(dev), cs_d,
                                     slots.to(dev), init.to(dev),
@@ -618,19 +618,24 @@ def test_delta_rule_kernels_match_reference(H, G, Dk, Dv, taps, dtype, off):
         o = ops.delta_rule_varlen(
             conv[:, :gk], conv[:, gk:2 * gk], conv[:, 2 * gk:],
             abd[:, :H], abd[:, H:], A_log.to(dev), dtb.to(dev), st_d,
-            slots.to(dev), init.to(dev), qsl.to(dev), Dk ** -0.5)
+            slots.to(dev), init.to(dev), qsl.to(dev), Dk ** -0.5, mql)
         out = ops.rms_gate(o, z.to(dev), nw.to(dev), H, 1e-5, tdt)
         return (conv.float().cpu(), o.cpu(), out.float().cpu(),
                 cs_d.float().cpu(), st_d.cpu())
 
-    want, got = run("cpu"), run("cuda")
+    want = run("cpu")
     tol = 3e-2 if dtype == "bfloat16" else 1e-4
-    for name, a, b in zip(("conv", "o", "out", "conv_state", "state"),
-                          want, got):
-        scale = max(1.0, a.abs().max().item())
-        assert (a - b).abs().max().item() < tol * scale, name
-    # untouched slots stay as they were
-    assert torch.equal(got[4][2], st[2]) and torch.equal(got[4][6], st[6])
+    # 0: LDS-tiled recurrence (batches with portions); 1: the register
+    # form decode-only batches take (valid for any portion length)
+    for mql in (0, 1):
+        got = run("cuda", mql)
+        for name, a, b in zip(("conv", "o", "out", "conv_state", "state"),
+                              want, got):
+            scale = max(1.0, a.abs().max().item())
+            assert (a - b).abs().max().item() < tol * scale, (name, mql)
+        # untouched slots stay as they were
+        assert torch.equal(got[4][2], st[2])
+        assert torch.equal(got[4][6], st[6])
 
 
 @pytest.mark.gpu
