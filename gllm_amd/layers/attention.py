@@ -128,3 +128,74 @@ class WindowAttention(nn.Module):
             q, gate, k_cache, v_cache, fctx.block_table, fctx.seq_lens,
             fctx.query_start_loc, self.scale, self.window,
             self.keep_first, self.sink, fctx.max_query_len)
+
+
+class TalkingHeadsAttention(nn.Module):
+    """Paged causal attention whose heads talk before the softmax.
+
+    * keys double as values: the cache of this layer holds the
+      normalised, rotated keys (K side) and the keys as projected (V
+      side); there is no value projection
+    * q and k are rotated (``rotary``: layers.rotary.HalfRotary /
+      PairRotary or None) and then brought to unit RMS per head, with no
+      learned weight, inside one fused kernel that also writes the cache
+    * the H per-head score planes scale * q_g . k are mixed by ``talk``
+      [H, H] (s'_h = sum_g talk[h, g] s_g) before masking and softmax
+    * ``sink`` [H]: exp(sink_h) joins head h's softmax denominator
+
+    ``talk`` and ``sink`` are fp32 parameters (scores and softmax run in
+    fp32 whatever the model dtype is). Any GQA ratio, any head size.
+    """
+
+    def __init__(self, layer_idx: int, num_heads: int, num_kv_heads: int,
+                 head_dim: int, scale: float, eps: float,
+                 rotary: Optional[nn.Module] = None, sink: bool = True):
+        super().__init__()
+        assert num_heads % num_kv_heads == 0
+        self.layer_idx = layer_idx
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.scale = scale
+        self.eps = eps
+        self.rotary = rotary
+        self.talk = nn.Parameter(torch.eye(num_heads, dtype=torch.float32),
+                                 requires_grad=False)
+        if sink:
+            self.sink = nn.Parameter(
+                torch.zeros(num_heads, dtype=torch.float32),
+                requires_grad=False)
+        else:
+            self.register_parameter("sink", None)
+        self._no_rot = None
+
+    def _freqs(self, device):
+        r = self.rotary
+        if r is not None:
+            return r.freqs, r.mag, r.rot_dims, \
+                bool(getattr(r, "half_layout", False))
+        if self._no_rot is None or self._no_rot.device != device:
+            self._no_rot = torch.zeros(1, dtype=torch.float64, device=device)
+        return self._no_rot, 1.0, 0, False
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor,
+                fctx: ForwardContext,
+                layer_idx: Optional[int] = None) -> torch.Tensor:
+        """q [T, H*D], k [T, G*D] (row views of a merged projection are
+        fine). ``layer_idx`` overrides the cache index (a layer that
+        runs several times keeps one cache per run). Returns [T, H*D]."""
+        T = q.shape[0]
+        H, G, D = self.num_heads, self.num_kv_heads, self.head_dim
+        if fctx.is_profile_run:
+            return q.new_zeros(T, H * D)
+        idx = self.layer_idx if layer_idx is None else layer_idx
+        k_cache, v_cache = fctx.k_caches[idx], fctx.v_caches[idx]
+        freqs, mag, rot_dims, half = self._freqs(q.device)
+        ops.qk_norm_rope_store(
+            q, k, k, None, None, fctx.positions, fctx.slot_mapping, freqs,
+            mag, rot_dims, k_cache, v_cache, H, G, D, D, self.eps,
+            half_layout=half, norm_last=True)
+        return ops.talking_attention(
+            q, k_cache, v_cache, fctx.block_table, fctx.seq_lens,
+            fctx.query_start_loc, self.scale, self.talk, self.sink,
+            fctx.max_query_len)

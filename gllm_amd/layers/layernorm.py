@@ -47,7 +47,8 @@ class GemmaRMSNorm(nn.Module):
 
 
 class LayerNorm(nn.Module):
-    """LayerNorm with weight and bias over an fp32 residual stream.
+    """LayerNorm with weight and (optional) bias over an fp32 residual
+    stream.
 
     Sandwich-norm decoders (a norm before and after every sublayer) keep
     the stream in fp32 while sublayers run in the model dtype:
@@ -56,27 +57,46 @@ class LayerNorm(nn.Module):
     * ``norm.add_into(x, y, nxt)``      x += LN(y) in place and, when
       ``nxt`` (the next sublayer's pre-norm) is given, returns nxt(x) —
       one fused launch per boundary (ops.residual_layernorm)
+    * ``norm.add_into(x, y, nxt, gate=g)``  the same with the sublayer
+      result gated first: x += LN(y * sigmoid(g))
 
-    The bias parameter is named ``bias``; checkpoints that store it
-    under another name map it in the model's load_weights.
+    The bias parameter is named ``bias`` (None with ``bias=False``);
+    checkpoints that store it under another name map it in the model's
+    load_weights.
     """
 
     def __init__(self, hidden_size: int, eps: float = 1e-5,
-                 params_dtype=None):
+                 params_dtype=None, bias: bool = True):
         super().__init__()
         dtype = params_dtype or torch.get_default_dtype()
         self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype),
                                    requires_grad=False)
-        self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=dtype),
-                                 requires_grad=False)
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=dtype),
+                                     requires_grad=False)
+        else:
+            self.register_parameter("bias", None)
         self.eps = eps
+        self._w32 = None
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.layernorm_f32(x, self.weight, self.bias, self.eps,
                                  self.weight.dtype)
 
+    def forward_f32(self, x: torch.Tensor) -> torch.Tensor:
+        """LN(x) kept in fp32 (a norm whose result IS the residual
+        stream, e.g. right after the embedding)."""
+        if self.weight.dtype == torch.float32:
+            return self.forward(x)
+        if self._w32 is None or self._w32[0].device != x.device:
+            self._w32 = (self.weight.float(), None if self.bias is None
+                         else self.bias.float())
+        return ops.layernorm_f32(x, self._w32[0], self._w32[1], self.eps,
+                                 torch.float32)
+
     def add_into(self, x: torch.Tensor, y: torch.Tensor,
-                 nxt: Optional["LayerNorm"] = None):
+                 nxt: Optional["LayerNorm"] = None,
+                 gate: Optional[torch.Tensor] = None):
         pre = (nxt.weight, nxt.bias) if nxt is not None else None
         return ops.residual_layernorm(x, y, self.weight, self.bias,
-                                      self.eps, pre)
+                                      self.eps, pre, gate)

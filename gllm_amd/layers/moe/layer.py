@@ -22,8 +22,19 @@ from gllm_amd.parallel import (get_ep_rank, get_ep_size, get_tp_rank,
 class FusedMoE(nn.Module):
     def __init__(self, num_experts: int, top_k: int, hidden_size: int,
                  intermediate_size: int, renormalize: bool = True,
-                 use_ep: bool = False, params_dtype=None):
+                 use_ep: bool = False, params_dtype=None,
+                 activation: str = "silu_glu",
+                 fp32_routing_weights: bool = False):
+        """``activation``: "silu_glu" — gated experts, w13 holds gate
+        and up rows, act = silu(gate) * up; "relu2" — ungated experts,
+        w13 holds the up rows only, act = max(z, 0)^2.
+        ``fp32_routing_weights``: keep the routing weights in fp32 up to
+        the weighted sum instead of rounding them to the model dtype."""
         super().__init__()
+        assert activation in ("silu_glu", "relu2")
+        self.activation = activation
+        self.gated = activation == "silu_glu"
+        self.fp32_routing_weights = fp32_routing_weights
         dtype = params_dtype or torch.get_default_dtype()
         self.num_experts = num_experts
         self.top_k = top_k
@@ -47,7 +58,8 @@ class FusedMoE(nn.Module):
 
         I = self.intermediate_per_rank
         self.w13_weight = nn.Parameter(
-            torch.empty(self.num_local_experts, 2 * I, hidden_size,
+            torch.empty(self.num_local_experts,
+                        (2 if self.gated else 1) * I, hidden_size,
                         dtype=dtype), requires_grad=False)
         self.w2_weight = nn.Parameter(
             torch.empty(self.num_local_experts, hidden_size, I, dtype=dtype),
@@ -69,7 +81,9 @@ class FusedMoE(nn.Module):
         return None
 
     def _load_w13(self, param, loaded, expert_id: int, shard_id: int):
-        """shard_id: 0 = gate (w1), 1 = up (w3)."""
+        """shard_id: 0 = gate (w1), 1 = up (w3); ungated experts have
+        the up rows only (shard 0)."""
+        assert self.gated or shard_id == 0
         lid = self._local_expert(expert_id)
         if lid is None:
             return
@@ -105,7 +119,9 @@ class FusedMoE(nn.Module):
         from gllm_amd.parallel import get_dp_size
         if self.use_ep and get_dp_size() > 1:
             return self._forward_dp(x, weights, ids)
-        out = self._expert_loop(x, weights.to(x.dtype), ids)
+        if not self.fp32_routing_weights:
+            weights = weights.to(x.dtype)
+        out = self._expert_loop(x, weights, ids)
         if self.use_ep:
             from gllm_amd.parallel.state import ep_all_reduce
             out = ep_all_reduce(out)
@@ -161,7 +177,8 @@ class FusedMoE(nn.Module):
                 return ops.fused_moe(
                     x.contiguous(), self.w13_weight, self.w2_weight,
                     weights, ids, expert_start=self.expert_start,
-                    num_global_experts=self.num_experts)
+                    num_global_experts=self.num_experts,
+                    activation=self.activation)
             if (self.fp8_block == (128, 128)
                     and x.shape[1] % 128 == 0
                     and self.intermediate_per_rank % 128 == 0):
@@ -187,6 +204,8 @@ class FusedMoE(nn.Module):
                     expert_start=self.expert_start)
         T = x.shape[0]
         out = torch.zeros_like(x)
+        acc = torch.zeros(x.shape, dtype=torch.float32, device=x.device) \
+            if weights.dtype != x.dtype else None
         flat_ids = ids.long().flatten()                    # [T*K]
         flat_rows = torch.arange(T, device=x.device).repeat_interleave(
             self.top_k)
@@ -210,10 +229,16 @@ class FusedMoE(nn.Module):
                 w13, w2 = self._dequant_expert(lid, x.dtype, x.device)
             else:
                 w13, w2 = self.w13_weight[lid], self.w2_weight[lid]
-            h = ops.silu_and_mul(ops.linear(xe, w13))
+            h = ops.linear(xe, w13)
+            h = ops.silu_and_mul(h) if self.gated else ops.relu2(h)
             ye = ops.linear(h, w2)
             w = flat_w[sel].unsqueeze(-1)
-            out.index_add_(0, rows, ye * w)
+            if w.dtype != ye.dtype:       # fp32 routing weights
+                acc.index_add_(0, rows, ye.float() * w)
+            else:
+                out.index_add_(0, rows, ye * w)
+        if acc is not None:
+            return acc.to(x.dtype)
         return out
 
     def _dequant_expert(self, lid: int, dtype, device):

@@ -234,3 +234,26 @@ class PairRotary(nn.Module):
             freqs = freqs / factor * ramp + freqs * (1.0 - ramp)
             self.mag = 0.1 * math.log(factor) + 1.0
         self.register_buffer("freqs", freqs, persistent=False)
+
+
+class HalfRotary(nn.Module):
+    """Rotate-half rotary on the first ``rot_dims`` dims of a head:
+    dimension i pairs with i + rot_dims/2 (i < rot_dims/2), frequency
+    base^(-2i/rot_dims); the remaining dims pass through.
+
+    Like PairRotary it holds only the fp64 per-pair frequencies; the
+    fused q/k kernel (ops.qk_norm_rope_store with ``half_layout``) forms
+    position * frequency in fp64, so no position table is sized.
+    """
+
+    half_layout = True
+    mag = 1.0
+
+    def __init__(self, rot_dims: int, base: float):
+        super().__init__()
+        assert rot_dims % 2 == 0
+        self.rot_dims = rot_dims
+        i = torch.arange(rot_dims // 2, dtype=torch.float64)
+        freqs = torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                          -2.0 * i / max(rot_dims, 1))
+        self.register_buffer("freqs", freqs, persistent=False)

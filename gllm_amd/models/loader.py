@@ -34,8 +34,10 @@ def get_arch_registry():
                                           Qwen3VLMoeForCausalLM,
                                           Qwen3_5VLForCausalLM)
     from gllm_amd.models.sudevik import SudevikForCausalLM
+    from gllm_amd.models.gukirax import GukiraxForCausalLM
     return {
         "Sudevik": SudevikForCausalLM,
+        "Gukirax": GukiraxForCausalLM,
         "Qwen2VLForConditionalGeneration": Qwen2VLForCausalLM,
         "Qwen2_5_VLForConditionalGeneration": Qwen2VLForCausalLM,
         "Qwen3VLForConditionalGeneration": Qwen3VLForCausalLM,

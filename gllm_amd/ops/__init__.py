@@ -207,8 +207,11 @@ def grouped_topk(scores, topk, n_group, topk_group, renormalize=True,
 def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
               topk_weights: torch.Tensor, topk_ids: torch.Tensor,
               expert_start: int = 0,
-              num_global_experts: Optional[int] = None) -> torch.Tensor:
+              num_global_experts: Optional[int] = None,
+              activation: str = "silu_glu") -> torch.Tensor:
     """Grouped-GEMM fused MoE on the gfx950 kernels (GPU, bf16).
+    ``activation``: "silu_glu" (w13 = gate | up rows) or "relu2"
+    (ungated experts, w13 = up rows only, act = max(z, 0)^2).
 
     Reference fused_experts_impl (fused_moe_triton/fused_moe.py:779):
     align -> GEMM1 -> silu_and_mul -> GEMM2 (weighted scatter) -> sum.
@@ -219,7 +222,6 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
     """
     T, K = x.shape
     E_local, two_i, _ = w13.shape
-    inter = two_i // 2
     topk = topk_ids.shape[1]
     n_pairs = T * topk
     # tile heuristic: match block_m to the expected rows per expert so
@@ -249,7 +251,7 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
     inter1 = torch.empty(rows_pad, two_i, dtype=x.dtype, device=dev)
     k.moe_gemm(inter1, x, w13, sorted_ids, expert_blocks, n_post, None,
                n_pairs, topk, gemm_m, False)
-    act = silu_and_mul(inter1)
+    act = relu2(inter1) if activation == "relu2" else silu_and_mul(inter1)
     # zero-filled: pairs routed to non-local experts (EP shards) or to
     # the DP padding id -1 are dropped by the align kernel and must
     # contribute zeros
@@ -387,7 +389,6 @@ def fused_moe_fp8(x: torch.Tensor, w13: torch.Tensor, w13_scale,
     block-scale fp8 GEMMs; expert weights stay e4m3-resident."""
     T, K = x.shape
     E_local, two_i, _ = w13.shape
-    inter = two_i // 2
     topk = topk_ids.shape[1]
     n_pairs = T * topk
     # same tile heuristic as the bf16 path (164 = BM64 x BN256 prefill)
@@ -417,7 +418,7 @@ def fused_moe_fp8(x: torch.Tensor, w13: torch.Tensor, w13_scale,
                    w13.view(torch.uint8), w13_scale.contiguous(),
                    sorted_ids, expert_blocks, n_post, None, n_pairs, topk,
                    gemm_m, False)
-    act = silu_and_mul(inter1)
+    act = relu2(inter1) if activation == "relu2" else silu_and_mul(inter1)
     actq, act_s = per_token_group_quant_fp8(act)
     pair_out = x.new_zeros(n_pairs, K)
     k.moe_gemm_fp8(pair_out, actq.view(torch.uint8), act_s,
@@ -551,7 +552,7 @@ def fused_moe_int4(x: torch.Tensor, w13_c, w13_sb, w2_c, w2_sb,
     k.moe_gemm_int4(inter1, x.contiguous(), w13_c, w13_sb, sorted_ids,
                     expert_blocks, n_post, None, n_pairs, topk, block_m,
                     False)
-    act = silu_and_mul(inter1)
+    act = relu2(inter1) if activation == "relu2" else silu_and_mul(inter1)
     pair_out = x.new_zeros(n_pairs, K)
     k.moe_gemm_int4(pair_out, act, w2_c, w2_sb, sorted_ids,
                     expert_blocks, n_post,
@@ -736,10 +737,11 @@ def linear(x: torch.Tensor, w: torch.Tensor,
 
 
 # --------------------------------------------------------------- layer norm
-def layernorm_f32(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor,
-                  eps: float, dtype) -> torch.Tensor:
-    """h = LayerNorm(x) with weight and bias; x is the fp32 residual
-    stream, h comes out in the model dtype."""
+def layernorm_f32(x: torch.Tensor, w: torch.Tensor, b, eps: float,
+                  dtype) -> torch.Tensor:
+    """h = LayerNorm(x) with weight and optional bias (``b`` None =
+    weight only); x is the fp32 residual stream, h comes out in
+    ``dtype`` (the dtype of w and b)."""
     if x.is_cuda:
         out = torch.empty(x.shape, dtype=dtype, device=x.device)
         _seq_kernels().layernorm_f32(out, x, w, b, eps)
@@ -748,38 +750,49 @@ def layernorm_f32(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor,
 
 
 def residual_layernorm(x: torch.Tensor, y: torch.Tensor, w_post, b_post,
-                       eps: float, pre=None):
+                       eps: float, pre=None, gate=None):
     """x (fp32, in place) += LN_post(y); with ``pre`` = (weight, bias)
     also returns LN_pre(x) in y's dtype — one launch per layer boundary
-    of a sandwich-norm decoder."""
+    of a sandwich-norm decoder. Biases may be None. ``gate`` ([rows,
+    width] logits, row views allowed): LN_post sees y * sigmoid(gate),
+    the product formed in fp32 inside the same launch."""
     if x.is_cuda:
         h = None
         if pre is not None:
             h = torch.empty(x.shape, dtype=y.dtype, device=x.device)
             _seq_kernels().residual_layernorm(x, y, w_post, b_post, h,
-                                              pre[0], pre[1], eps)
+                                              pre[0], pre[1], eps, gate)
         else:
             _seq_kernels().residual_layernorm(x, y, w_post, b_post, None,
-                                              None, None, eps)
+                                              None, None, eps, gate)
         return h
-    return torch_ref.residual_layernorm(x, y, w_post, b_post, eps, pre)
+    return torch_ref.residual_layernorm(x, y, w_post, b_post, eps, pre,
+                                        gate)
 
 
 # --------------------------------------------------------------- windowed attn
 def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
-                       mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps):
-    """Fused per-head q/k RMS norm, interleaved-pair rotary (per-pair
-    frequency table ``freqs`` fp64, cos/sin scaled by ``mag``) and paged
-    K/V store. q [T, H*D] is updated in place (may be a column slice of
-    a merged projection); k/v None = the layer reads another's cache."""
+                       mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
+                       half_layout=False, norm_last=False):
+    """Fused per-head q/k RMS norm, rotary (per-pair frequency table
+    ``freqs`` fp64, cos/sin scaled by ``mag``) and paged K/V store.
+    q [T, H*D] is updated in place (may be a column slice of a merged
+    projection); k/v None = the layer reads another's cache.
+
+    ``q_w``/``k_w`` None: unit-RMS heads without a weight.
+    ``half_layout``: dimension i rotates with i + rot_dims/2 (the
+    default pairs 2i with 2i+1). ``norm_last``: rotate, then norm.
+    ``v`` may be ``k`` itself (values = keys as projected)."""
     if q.is_cuda:
         _seq_kernels().qk_norm_rope_store(
             q, k, v, q_w, k_w, positions, slot_mapping, freqs, mag,
-            rot_dims, k_cache, v_cache, H, G, D, Dv, eps)
+            rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
+            bool(half_layout), bool(norm_last))
         return
     torch_ref.qk_norm_rope_store(q, k, v, q_w, k_w, positions,
                                  slot_mapping, freqs, mag, rot_dims,
-                                 k_cache, v_cache, H, G, D, Dv, eps)
+                                 k_cache, v_cache, H, G, D, Dv, eps,
+                                 half_layout, norm_last)
 
 
 def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
@@ -822,6 +835,54 @@ def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
                                       block_table, seq_lens,
                                       query_start_loc, scale, window,
                                       keep_first, sink)
+
+
+# --------------------------------------------------------------- talking heads
+def talking_attention(q, k_cache, v_cache, block_table, seq_lens,
+                      query_start_loc, scale, talk, sink=None,
+                      max_query_len=0) -> torch.Tensor:
+    """Ragged paged causal attention with cross-head score mixing:
+    s_g = scale * q_g . k_kv(g) for all H heads, s'_h = sum_g
+    talk[h, g] s_g, softmax over the keys per head with exp(sink[h])
+    added to the denominator (``sink`` None: plain softmax), output
+    head h = weights . v_kv(h). K [pages, page, G, D], V [.., Dv];
+    talk [H, H] and sink [H] fp32. Returns [T, H*Dv].
+
+    All heads of a query are handled together (the mix couples them).
+    bf16 batches with prompt portions and D == Dv a multiple of 32
+    run the MFMA tile kernel; bf16 decode-only batches the split-KV
+    kernel; fp32 and other shapes the generic kernel."""
+    if q.is_cuda:
+        T = q.shape[0]
+        D, Dv = k_cache.shape[3], v_cache.shape[3]
+        H = q.shape[1] // D
+        out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+        _seq_kernels().talking_attention(
+            out, q, k_cache, v_cache, block_table, seq_lens,
+            query_start_loc, scale, talk, sink, max_query_len)
+        return out
+    return torch_ref.talking_attention(q, k_cache, v_cache, block_table,
+                                       seq_lens, query_start_loc, scale,
+                                       talk, sink)
+
+
+# --------------------------------------------------------------- activations
+def xielu(x: torch.Tensor, a_pos: float, a_neg: float) -> torch.Tensor:
+    """xIELU: z > 0 -> a_pos z^2 + z/2, else a_neg (e^z - 1 - z) + z/2."""
+    if x.is_cuda:
+        out = torch.empty_like(x)
+        _seq_kernels().xielu(out, x, a_pos, a_neg)
+        return out
+    return torch_ref.xielu(x, a_pos, a_neg)
+
+
+def relu2(x: torch.Tensor) -> torch.Tensor:
+    """max(x, 0)^2."""
+    if x.is_cuda:
+        out = torch.empty_like(x)
+        _seq_kernels().relu2(out, x)
+        return out
+    return torch_ref.relu2(x)
 
 
 # --------------------------------------------------------------- delta rule

@@ -1,0 +1,355 @@
+// Talking-heads attention over the paged KV cache, gfx950.
+//
+// Causal attention whose H per-head score planes are mixed across heads
+// before the softmax:
+//
+//   s_g(i, j)  = scale * q_g(i) . k_kv(g)(j)          all heads g
+//   s'_h(i, j) = sum_g talk[h, g] * s_g(i, j)
+//   w_h(i, .)  = exp(s'_h) / (sum_{j <= i} exp(s'_h) + exp(sink_h))
+//   o_h(i)     = sum_j w_h(i, j) * v_kv(h)(j)
+//
+// The mix couples the heads, so one workgroup owns ALL heads of its
+// queries. Scores, the mix, softmax statistics and the sink are fp32
+// whatever the I/O type T (bf16 or fp32) is.
+//
+//   talking_attention_kernel   any D, Dv, H, G, page size, dtype: one
+//       workgroup per (query token, key split); 64-key tiles: raw scores
+//       -> LDS, mix + online softmax (one wave per head), P.V with the
+//       accumulators in registers. Decode-only batches split the keys
+//       over several workgroups (partials + talking_merge_kernel).
+//   talking_mfma_kernel        bf16, D == Dv a multiple of 32, batches
+//       with prompt portions: 32 queries of one sequence per workgroup,
+//       K/V tiles of 32 keys staged through LDS, S^T = K Q^T and
+//       O^T = V^T P^T on 32x32x8 MFMA; the raw score planes of all heads
+//       pass through LDS for the fp32 mix.
+
+#include <torch/extension.h>
+#include <ATen/cuda/CUDAContext.h>
+#include "common.h"
+
+namespace {
+
+constexpr int TK_BLOCK = 256;
+constexpr int TK_KEYS = 64;   // keys per tile = one wave of scores
+
+// which sequence owns flat token t: largest b with qsl[b] <= t
+DEV_INLINE int owner_of(const int *__restrict__ qsl, int B, int t) {
+  int lo = 0, hi = B - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (qsl[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+template <typename T>
+DEV_INLINE float dot_row(const float *__restrict__ qs,
+                         const T *__restrict__ kr, int D) {
+  float dot = 0.f;
+  if (sizeof(T) == 2 && D % 8 == 0) {
+    for (int d = 0; d < D; d += 8) {
+      float kf[8];
+      unpack8<T>(*reinterpret_cast<const shortx8 *>(kr + d), kf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot += qs[d + e] * kf[e];
+    }
+  } else if (sizeof(T) == 4 && D % 4 == 0) {
+    for (int d = 0; d < D; d += 4) {
+      const floatx4 kf = *reinterpret_cast<const floatx4 *>(kr + d);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dot += qs[d + e] * kf[e];
+    }
+  } else {
+    for (int d = 0; d < D; ++d) dot += qs[d] * ScalarOps<T>::to_f32(kr[d]);
+  }
+  return dot;
+}
+
+// grid (tokens, splits). NACC = ceil(H * Dv / 256) rounded up to a power
+// of two: output element o = tid + c * 256 (head o / Dv, column o % Dv).
+template <typename T, int NACC>
+__global__ __launch_bounds__(TK_BLOCK) void talking_attention_kernel(
+    T *__restrict__ out, float *__restrict__ part_acc,
+    float *__restrict__ part_ml, const T *__restrict__ q, long q_stride,
+    const T *__restrict__ k_cache, const T *__restrict__ v_cache,
+    const int *__restrict__ block_table, int bt_stride,
+    const int *__restrict__ seq_lens, const int *__restrict__ qsl, int B,
+    int H, int G, int D, int Dv, int page, float scale,
+    const float *__restrict__ talk, const float *__restrict__ sink,
+    int splits) {
+  extern __shared__ float smem[];
+  const int HD = (H * D + 3) & ~3;
+  float *qs = smem;                    // [H * D]
+  float *tk = qs + HD;                 // [H * H]
+  float *sraw = tk + ((H * H + 3) & ~3);  // [H][64] raw scores
+  float *pp = sraw + H * TK_KEYS;      // [H][64] softmax numerators
+  float *mrun = pp + H * TK_KEYS;      // [H] running max
+  float *lrun = mrun + H;              // [H] running sum
+  float *corr = lrun + H;              // [H] rescale of this tile
+  long *rows = reinterpret_cast<long *>(
+      smem + ((HD + ((H * H + 3) & ~3) + 2 * H * TK_KEYS + 3 * H + 1) & ~1));
+
+  const int t = blockIdx.x, sp = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = owner_of(qsl, B, t);
+  const int i = seq_lens[b] - (qsl[b + 1] - t);   // position of row t
+  const int total = i + 1;                         // keys 0..i
+  const int *bt = block_table + (long)b * bt_stride;
+  const int rep = H / G;
+
+  const int tiles = (total + TK_KEYS - 1) / TK_KEYS;
+  const int tiles_per = (tiles + splits - 1) / splits;
+  const int j0 = sp * tiles_per * TK_KEYS;
+  const int j1 = min(total, j0 + tiles_per * TK_KEYS);
+
+  for (int d = tid; d < H * D; d += TK_BLOCK)
+    qs[d] = ScalarOps<T>::to_f32(q[(long)t * q_stride + d]);
+  for (int d = tid; d < H * H; d += TK_BLOCK) tk[d] = talk[d];
+  for (int h = tid; h < H; h += TK_BLOCK) {
+    mrun[h] = -INFINITY;
+    lrun[h] = 0.f;
+  }
+  float acc[NACC];
+#pragma unroll
+  for (int c = 0; c < NACC; ++c) acc[c] = 0.f;
+
+  for (int base = j0; base < j1; base += TK_KEYS) {
+    const int n_tile = min(TK_KEYS, j1 - base);
+    __syncthreads();   // q/talk staged; last tile's pp/rows are done with
+    if (tid < TK_KEYS) {
+      const int j = base + tid;
+      rows[tid] = tid < n_tile ? (long)bt[j / page] * page + j % page : 0;
+    }
+    __syncthreads();
+    // raw scores: lane = key, wave strides over the heads
+    for (int h = wave; h < H; h += TK_BLOCK / 64) {
+      float s = 0.f;
+      if (lane < n_tile)
+        s = dot_row<T>(qs + h * D, k_cache + (rows[lane] * G + h / rep) * D,
+                       D) * scale;
+      sraw[h * TK_KEYS + lane] = s;
+    }
+    __syncthreads();
+    // mix + online softmax: a wave owns head h for this tile
+    for (int h = wave; h < H; h += TK_BLOCK / 64) {
+      float s = 0.f;
+      for (int g = 0; g < H; ++g) s += tk[h * H + g] * sraw[g * TK_KEYS + lane];
+      if (lane >= n_tile) s = -INFINITY;
+      const float m_old = mrun[h];
+      const float m_new = fmaxf(m_old, wave_reduce_max(s));
+      const float p = lane < n_tile ? expf(s - m_new) : 0.f;
+      const float psum = wave_reduce_sum(p);
+      const float c = m_old == -INFINITY ? 0.f : expf(m_old - m_new);
+      pp[h * TK_KEYS + lane] = p;
+      if (lane == 0) {
+        mrun[h] = m_new;
+        lrun[h] = lrun[h] * c + psum;
+        corr[h] = c;
+      }
+    }
+    __syncthreads();
+    // P.V
+#pragma unroll
+    for (int c = 0; c < NACC; ++c) {
+      const int o = tid + c * TK_BLOCK;
+      if (o < H * Dv) {
+        const int h = o / Dv, d = o - h * Dv;
+        const float *ph = pp + h * TK_KEYS;
+        const T *vb = v_cache + (long)(h / rep) * Dv + d;
+        float a = acc[c] * corr[h];
+        for (int jj = 0; jj < n_tile; ++jj)
+          a += ph[jj] * ScalarOps<T>::to_f32(vb[rows[jj] * G * Dv]);
+        acc[c] = a;
+      }
+    }
+  }
+  __syncthreads();
+  if (splits == 1) {
+#pragma unroll
+    for (int c = 0; c < NACC; ++c) {
+      const int o = tid + c * TK_BLOCK;
+      if (o < H * Dv) {
+        const int h = o / Dv;
+        float m = mrun[h], l = lrun[h], a = acc[c];
+        if (sink != nullptr) {
+          const float sk = sink[h];
+          const float M = fmaxf(m, sk);
+          const float w = expf(m - M);
+          l = l * w + expf(sk - M);
+          a *= w;
+        }
+        out[(long)t * H * Dv + o] = ScalarOps<T>::from_f32(a / l);
+      }
+    }
+  } else {
+    const long pbase = (long)t * splits + sp;
+#pragma unroll
+    for (int c = 0; c < NACC; ++c) {
+      const int o = tid + c * TK_BLOCK;
+      if (o < H * Dv) part_acc[pbase * H * Dv + o] = acc[c];
+    }
+    for (int h = tid; h < H; h += TK_BLOCK) {
+      part_ml[(pbase * H + h) * 2] = mrun[h];
+      part_ml[(pbase * H + h) * 2 + 1] = lrun[h];
+    }
+  }
+}
+
+// grid (tokens): combine the key splits of one query, sink included
+template <typename T>
+__global__ __launch_bounds__(TK_BLOCK) void talking_merge_kernel(
+    T *__restrict__ out, const float *__restrict__ part_acc,
+    const float *__restrict__ part_ml, const float *__restrict__ sink, int H,
+    int Dv, int splits) {
+  const int t = blockIdx.x;
+  for (int o = threadIdx.x; o < H * Dv; o += TK_BLOCK) {
+    const int h = o / Dv;
+    float M = sink != nullptr ? sink[h] : -INFINITY;
+    for (int s = 0; s < splits; ++s)
+      M = fmaxf(M, part_ml[(((long)t * splits + s) * H + h) * 2]);
+    float l = sink != nullptr ? expf(sink[h] - M) : 0.f;
+    float a = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const long pb = (long)t * splits + s;
+      const float m = part_ml[(pb * H + h) * 2];
+      if (m == -INFINITY) continue;     // a split with no keys
+      const float w = expf(m - M);
+      l += part_ml[(pb * H + h) * 2 + 1] * w;
+      a += part_acc[pb * H * Dv + o] * w;
+    }
+    out[(long)t * H * Dv + o] = ScalarOps<T>::from_f32(a / l);
+  }
+}
+
+bool rows_ok2(const torch::Tensor &t) {
+  return t.dim() == 2 && t.stride(1) == 1;
+}
+
+}  // namespace
+
+bool talking_attention_mfma(torch::Tensor &out, torch::Tensor &q,
+                            torch::Tensor &k_cache, torch::Tensor &v_cache,
+                            torch::Tensor &block_table,
+                            torch::Tensor &seq_lens,
+                            torch::Tensor &query_start_loc, double scale,
+                            torch::Tensor &talk, const float *sink,
+                            long max_query_len);
+
+void talking_attention(torch::Tensor out, torch::Tensor q,
+                       torch::Tensor k_cache, torch::Tensor v_cache,
+                       torch::Tensor block_table, torch::Tensor seq_lens,
+                       torch::Tensor query_start_loc, double scale,
+                       torch::Tensor talk, c10::optional<torch::Tensor> sink,
+                       long max_query_len) {
+  const long T = q.size(0);
+  if (T == 0) return;
+  const auto st = q.scalar_type();
+  TORCH_CHECK(q.is_cuda() && k_cache.dim() == 4 && v_cache.dim() == 4);
+  const int page = k_cache.size(1), G = k_cache.size(2), D = k_cache.size(3);
+  const int Dv = v_cache.size(3);
+  TORCH_CHECK(rows_ok2(q) && q.size(1) % D == 0);
+  const int H = q.size(1) / D;
+  TORCH_CHECK(G > 0 && H % G == 0,
+              "query heads must be a multiple of kv heads");
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.scalar_type() == st && v_cache.scalar_type() == st);
+  TORCH_CHECK(v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == page &&
+              v_cache.size(2) == G);
+  TORCH_CHECK(out.is_contiguous() && out.scalar_type() == st &&
+              out.numel() == T * H * Dv);
+  TORCH_CHECK(block_table.scalar_type() == at::kInt && block_table.dim() == 2 &&
+              block_table.stride(1) == 1);
+  TORCH_CHECK(seq_lens.scalar_type() == at::kInt && seq_lens.is_contiguous());
+  TORCH_CHECK(query_start_loc.scalar_type() == at::kInt &&
+              query_start_loc.is_contiguous());
+  const int B = seq_lens.numel();
+  TORCH_CHECK(query_start_loc.numel() >= B + 1 && block_table.size(0) >= B);
+  TORCH_CHECK(talk.is_cuda() && talk.scalar_type() == at::kFloat &&
+              talk.is_contiguous() && talk.numel() == (long)H * H,
+              "talk must be fp32 [H, H]");
+  const float *sp = nullptr;
+  if (sink.has_value()) {
+    TORCH_CHECK(sink->is_cuda() && sink->scalar_type() == at::kFloat &&
+                sink->is_contiguous() && sink->numel() == H,
+                "sink must be fp32 [H]");
+    sp = sink->data_ptr<float>();
+  }
+  TORCH_CHECK((long)H * Dv <= 32 * TK_BLOCK,
+              "talking_attention: heads * value size <= 8192");
+
+  if (st == at::kBFloat16 && max_query_len > 1 &&
+      talking_attention_mfma(out, q, k_cache, v_cache, block_table, seq_lens,
+                             query_start_loc, scale, talk, sp,
+                             max_query_len))
+    return;
+
+  // decode-only batches: spread the keys of each query over workgroups
+  // (fixed by the batch size alone, so a captured graph keeps its shape)
+  int splits = 1;
+  if (max_query_len == 1 && T < 512)
+    splits = (int)std::min<long>(16, (1024 + T - 1) / T);
+  torch::Tensor pacc, pml;
+  float *paccp = nullptr, *pmlp = nullptr;
+  if (splits > 1) {
+    auto opts = torch::TensorOptions().dtype(at::kFloat).device(q.device());
+    pacc = torch::empty({T, splits, (long)H * Dv}, opts);
+    pml = torch::empty({T, splits, (long)H, 2}, opts);
+    paccp = pacc.data_ptr<float>();
+    pmlp = pml.data_ptr<float>();
+  }
+  const int HD = (H * D + 3) & ~3, HH = (H * H + 3) & ~3;
+  const int nf = (HD + HH + 2 * H * TK_KEYS + 3 * H + 1) & ~1;
+  const size_t lds = (size_t)nf * sizeof(float) + TK_KEYS * sizeof(long);
+  TORCH_CHECK(lds <= 64 * 1024, "talking_attention: heads * dim too large");
+  int nacc = 1;
+  while (nacc * TK_BLOCK < H * Dv) nacc *= 2;
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(TT, N)                                                           \
+  hipLaunchKernelGGL((talking_attention_kernel<TT, N>), dim3(T, splits),     \
+                     dim3(TK_BLOCK), lds, stream, (TT *)out.data_ptr(),      \
+                     paccp, pmlp, (const TT *)q.data_ptr(),                  \
+                     (long)q.stride(0), (const TT *)k_cache.data_ptr(),      \
+                     (const TT *)v_cache.data_ptr(),                         \
+                     block_table.data_ptr<int>(), (int)block_table.stride(0), \
+                     seq_lens.data_ptr<int>(),                               \
+                     query_start_loc.data_ptr<int>(), B, H, G, D, Dv, page,  \
+                     (float)scale, talk.data_ptr<float>(), sp, splits)
+#define RUN_N(TT)                                                            \
+  switch (nacc) {                                                            \
+    case 1: RUN(TT, 1); break;                                               \
+    case 2: RUN(TT, 2); break;                                               \
+    case 4: RUN(TT, 4); break;                                               \
+    case 8: RUN(TT, 8); break;                                               \
+    case 16: RUN(TT, 16); break;                                             \
+    default: RUN(TT, 32); break;                                             \
+  }
+  if (st == at::kBFloat16) { RUN_N(__hip_bfloat16) }
+  else if (st == at::kFloat) { RUN_N(float) }
+  else TORCH_CHECK(false, "talking_attention: bf16 or fp32");
+#undef RUN_N
+#undef RUN
+  HIP_CHECK_KERNEL();
+  if (splits > 1) {
+    if (st == at::kBFloat16)
+      hipLaunchKernelGGL((talking_merge_kernel<__hip_bfloat16>), dim3(T),
+                         dim3(TK_BLOCK), 0, stream,
+                         (__hip_bfloat16 *)out.data_ptr(), paccp, pmlp, sp, H,
+                         Dv, splits);
+    else
+      hipLaunchKernelGGL((talking_merge_kernel<float>), dim3(T),
+                         dim3(TK_BLOCK), 0, stream, (float *)out.data_ptr(),
+                         paccp, pmlp, sp, H, Dv, splits);
+    HIP_CHECK_KERNEL();
+  }
+}
+
+// the MFMA tile form is added below this line
+bool talking_attention_mfma(torch::Tensor &out, torch::Tensor &q,
+                            torch::Tensor &k_cache, torch::Tensor &v_cache,
+                            torch::Tensor &block_table,
+                            torch::Tensor &seq_lens,
+                            torch::Tensor &query_start_loc, double scale,
+                            torch::Tensor &talk, const float *sink,
+                            long max_query_len) {
+  return false;
+}

@@ -4,12 +4,14 @@
 // and accumulation are fp32 always) and shape-generic: any per-head
 // query/key size D, value size Dv != D, any GQA ratio, any page size.
 //
-//   qk_norm_rope_store  per-head RMS norm of q and k (plain weight),
-//                       interleaved-pair rotary on the first rot_dims
-//                       dims with a per-pair frequency table (YaRN or
-//                       plain; angle = pos * f in fp64, so long
-//                       positions lose nothing), then q in place and
-//                       k, v scattered into the paged cache
+//   qk_norm_rope_store  per-head RMS norm of q and k (plain weight or
+//                       none), rotary on the first rot_dims dims with a
+//                       per-pair frequency table (YaRN or plain; angle =
+//                       pos * f in fp64, so long positions lose
+//                       nothing; pairs (2i, 2i+1) or, half layout,
+//                       (i, i + rot_dims/2)), norm before or after the
+//                       rotation, then q in place and k, v scattered
+//                       into the paged cache (v may be k as projected)
 //   window_attention    ragged batch (prompt portions beside single
 //                       decode tokens) over the paged cache: position i
 //                       sees j <= i with i - j < window or j < keep_first;
@@ -39,7 +41,7 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
     const T *__restrict__ k_w, const long *__restrict__ positions,
     const long *__restrict__ slot_mapping, const double *__restrict__ freqs,
     float mag, int rot_dims, T *__restrict__ k_cache, T *__restrict__ v_cache,
-    int H, int G, int D, int Dv, float eps) {
+    int H, int G, int D, int Dv, float eps, int half_layout, int norm_last) {
   extern __shared__ float buf[];
   const int t = blockIdx.x;
   const int y = blockIdx.y;
@@ -62,22 +64,36 @@ __global__ __launch_bounds__(QK_BLOCK) void qk_norm_rope_store_kernel(
     buf[i] = x;
     ss += x * x;
   }
-  ss = wave_reduce_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / D + eps);
   __syncthreads();
-  for (int i = lane; i < D; i += QK_BLOCK)
-    buf[i] = buf[i] * inv * ScalarOps<T>::to_f32(w[i]);
-  __syncthreads();
+  if (!norm_last) {
+    ss = wave_reduce_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / D + eps);
+    for (int i = lane; i < D; i += QK_BLOCK)
+      buf[i] = buf[i] * inv * (w ? ScalarOps<T>::to_f32(w[i]) : 1.0f);
+    __syncthreads();
+  }
   const double pos = (double)positions[t];
-  for (int p = lane; p < rot_dims / 2; p += QK_BLOCK) {
+  const int half = rot_dims / 2;
+  for (int p = lane; p < half; p += QK_BLOCK) {
     double sn, cs;
     sincos(pos * freqs[p], &sn, &cs);
     const float c = (float)cs * mag, s = (float)sn * mag;
-    const float a = buf[2 * p], b = buf[2 * p + 1];
-    buf[2 * p] = a * c - b * s;
-    buf[2 * p + 1] = b * c + a * s;
+    const int ia = half_layout ? p : 2 * p;
+    const int ib = half_layout ? p + half : 2 * p + 1;
+    const float a = buf[ia], b = buf[ib];
+    buf[ia] = a * c - b * s;
+    buf[ib] = b * c + a * s;
   }
   __syncthreads();
+  if (norm_last) {
+    ss = 0.f;
+    for (int i = lane; i < D; i += QK_BLOCK) ss += buf[i] * buf[i];
+    ss = wave_reduce_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / D + eps);
+    for (int i = lane; i < D; i += QK_BLOCK)
+      buf[i] = buf[i] * inv * (w ? ScalarOps<T>::to_f32(w[i]) : 1.0f);
+    __syncthreads();
+  }
   T *dst = is_q ? q + (long)t * q_stride + (long)y * D
                 : k_cache + (slot_mapping[t] * G + (y - H)) * D;
   for (int i = lane; i < D; i += QK_BLOCK)
@@ -232,19 +248,25 @@ bool rows_ok(const torch::Tensor &t) {
 }  // namespace
 
 void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
-                        c10::optional<torch::Tensor> v, torch::Tensor q_w,
+                        c10::optional<torch::Tensor> v,
+                        c10::optional<torch::Tensor> q_w,
                         c10::optional<torch::Tensor> k_w,
                         torch::Tensor positions, torch::Tensor slot_mapping,
                         torch::Tensor freqs, double mag, long rot_dims,
                         c10::optional<torch::Tensor> k_cache,
                         c10::optional<torch::Tensor> v_cache, long H, long G,
-                        long D, long Dv, double eps) {
+                        long D, long Dv, double eps, bool half_layout,
+                        bool norm_last) {
   const long T = q.size(0);
   if (T == 0) return;
   const auto st = q.scalar_type();
   TORCH_CHECK(q.is_cuda() && rows_ok(q) && q.size(1) == H * D);
-  TORCH_CHECK(q_w.scalar_type() == st && q_w.numel() == D &&
-              q_w.is_contiguous());
+  const void *qwp = nullptr;
+  if (q_w.has_value()) {
+    TORCH_CHECK(q_w->scalar_type() == st && q_w->numel() == D &&
+                q_w->is_contiguous());
+    qwp = q_w->data_ptr();
+  }
   TORCH_CHECK(positions.scalar_type() == at::kLong &&
               positions.is_contiguous() && positions.numel() >= T);
   TORCH_CHECK(freqs.scalar_type() == at::kDouble && freqs.is_contiguous() &&
@@ -257,13 +279,17 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
   void *kcp = nullptr, *vcp = nullptr;
   long ks = 0, vs = 0;
   if (own) {
-    TORCH_CHECK(v.has_value() && k_w.has_value() && k_cache.has_value() &&
-                v_cache.has_value());
+    TORCH_CHECK(v.has_value() && k_w.has_value() == q_w.has_value() &&
+                k_cache.has_value() && v_cache.has_value());
     TORCH_CHECK(rows_ok(*k) && k->size(0) == T && k->size(1) == G * D &&
                 k->scalar_type() == st);
     TORCH_CHECK(rows_ok(*v) && v->size(0) == T && v->size(1) == G * Dv &&
                 v->scalar_type() == st);
-    TORCH_CHECK(k_w->scalar_type() == st && k_w->numel() == D);
+    if (k_w.has_value()) {
+      TORCH_CHECK(k_w->scalar_type() == st && k_w->numel() == D &&
+                  k_w->is_contiguous());
+      kwp = k_w->data_ptr();
+    }
     TORCH_CHECK(k_cache->is_contiguous() && v_cache->is_contiguous() &&
                 k_cache->scalar_type() == st && v_cache->scalar_type() == st);
     TORCH_CHECK(k_cache->dim() == 4 && k_cache->size(2) == G &&
@@ -271,7 +297,7 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
                 v_cache->size(3) == Dv, "cache geometry mismatch");
     TORCH_CHECK(slot_mapping.scalar_type() == at::kLong &&
                 slot_mapping.is_contiguous() && slot_mapping.numel() >= T);
-    kp = k->data_ptr(); vp = v->data_ptr(); kwp = k_w->data_ptr();
+    kp = k->data_ptr(); vp = v->data_ptr();
     kcp = k_cache->data_ptr(); vcp = v_cache->data_ptr();
     ks = k->stride(0); vs = v->stride(0);
   }
@@ -281,12 +307,12 @@ void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
   hipLaunchKernelGGL((qk_norm_rope_store_kernel<TT>), dim3(T, gy),           \
                      dim3(QK_BLOCK), D * sizeof(float), stream,              \
                      (TT *)q.data_ptr(), (long)q.stride(0), (const TT *)kp,  \
-                     ks, (const TT *)vp, vs, (const TT *)q_w.data_ptr(),     \
+                     ks, (const TT *)vp, vs, (const TT *)qwp,                \
                      (const TT *)kwp, positions.data_ptr<long>(),            \
                      own ? slot_mapping.data_ptr<long>() : nullptr,          \
                      freqs.data_ptr<double>(), (float)mag, (int)rot_dims,    \
                      (TT *)kcp, (TT *)vcp, (int)H, (int)G, (int)D, (int)Dv,  \
-                     (float)eps)
+                     (float)eps, half_layout ? 1 : 0, norm_last ? 1 : 0)
   if (st == at::kBFloat16) RUN(__hip_bfloat16);
   else if (st == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "qk_norm_rope_store: bf16 or fp32");

@@ -1,24 +1,36 @@
 // Python bindings for the dtype-generic sequence-mixer kernels
 // (gllm_amd._kernels_seq): fp32-residual layer norm, windowed sink
-// attention, varlen gated delta rule, plus the grouped MoE GEMM and the
-// gated activations they are served with.
+// attention, talking-heads attention, varlen gated delta rule, plus the
+// grouped MoE GEMM and the activations they are served with.
 #include <torch/extension.h>
 
 void layernorm_f32(torch::Tensor out, torch::Tensor x, torch::Tensor w,
-                   torch::Tensor b, double eps);
+                   c10::optional<torch::Tensor> b, double eps);
 void residual_layernorm(torch::Tensor x, torch::Tensor y,
-                        torch::Tensor w_post, torch::Tensor b_post,
+                        torch::Tensor w_post,
+                        c10::optional<torch::Tensor> b_post,
                         c10::optional<torch::Tensor> h,
                         c10::optional<torch::Tensor> w_pre,
-                        c10::optional<torch::Tensor> b_pre, double eps);
+                        c10::optional<torch::Tensor> b_pre, double eps,
+                        c10::optional<torch::Tensor> gate);
 void qk_norm_rope_store(torch::Tensor q, c10::optional<torch::Tensor> k,
-                        c10::optional<torch::Tensor> v, torch::Tensor q_w,
+                        c10::optional<torch::Tensor> v,
+                        c10::optional<torch::Tensor> q_w,
                         c10::optional<torch::Tensor> k_w,
                         torch::Tensor positions, torch::Tensor slot_mapping,
                         torch::Tensor freqs, double mag, long rot_dims,
                         c10::optional<torch::Tensor> k_cache,
                         c10::optional<torch::Tensor> v_cache, long H, long G,
-                        long D, long Dv, double eps);
+                        long D, long Dv, double eps, bool half_layout,
+                        bool norm_last);
+void talking_attention(torch::Tensor out, torch::Tensor q,
+                       torch::Tensor k_cache, torch::Tensor v_cache,
+                       torch::Tensor block_table, torch::Tensor seq_lens,
+                       torch::Tensor query_start_loc, double scale,
+                       torch::Tensor talk, c10::optional<torch::Tensor> sink,
+                       long max_query_len);
+void xielu(torch::Tensor out, torch::Tensor x, double a_pos, double a_neg);
+void relu2(torch::Tensor out, torch::Tensor x);
 void window_attention(torch::Tensor out, torch::Tensor q,
                       c10::optional<torch::Tensor> gate,
                       torch::Tensor k_cache, torch::Tensor v_cache,
@@ -68,9 +80,15 @@ void moe_sum(torch::Tensor out, torch::Tensor pair_out, long topk);
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("layernorm_f32", &layernorm_f32, "h = LN(x fp32) in the model dtype");
   m.def("residual_layernorm", &residual_layernorm,
-        "x += LN_post(y); optionally h = LN_pre(x)");
+        "x += LN_post(y [* sigmoid(gate)]); optionally h = LN_pre(x)");
   m.def("qk_norm_rope_store", &qk_norm_rope_store,
-        "per-head q/k RMS norm + interleaved rotary + paged K/V store");
+        "per-head q/k RMS norm + rotary (pair or half layout, either "
+        "order) + paged K/V store");
+  m.def("talking_attention", &talking_attention,
+        "ragged paged causal attention with cross-head score mixing "
+        "and a per-head sink");
+  m.def("xielu", &xielu, "xIELU activation over row-strided input");
+  m.def("relu2", &relu2, "max(x, 0)^2 over row-strided input");
   m.def("window_attention", &window_attention,
         "ragged paged attention: window + kept first tokens + sink + gate");
   m.def("window_attention_mfma", &window_attention_mfma,

@@ -247,3 +247,97 @@ void reshape_and_cache(torch::Tensor k, torch::Tensor v,
                      page_size, k.stride(0), v.stride(0));
   HIP_CHECK_KERNEL();
 }
+
+// ------------------------------------------------------------------
+// Ungated feed-forward activations: out[r, i] = act(x[r, i]) for a
+// row-strided x (a column slice of a merged projection) and a
+// contiguous out. fp32 arithmetic whatever the I/O type is.
+namespace {
+
+struct XieluOp {
+  float a_pos, a_neg;
+  // z > 0: a_pos z^2 + z/2; z <= 0: a_neg (e^z - 1 - z) + z/2
+  DEV_INLINE float operator()(float z) const {
+    return z > 0.f ? a_pos * z * z + 0.5f * z
+                   : a_neg * (expm1f(z) - z) + 0.5f * z;
+  }
+};
+
+struct Relu2Op {
+  DEV_INLINE float operator()(float z) const {
+    const float r = fmaxf(z, 0.f);
+    return r * r;
+  }
+};
+
+template <typename T, typename Op, bool VEC>
+__global__ __launch_bounds__(256) void unary_rows_kernel(
+    T *__restrict__ out, const T *__restrict__ x, long x_stride, long rows,
+    int n, Op op) {
+  if (VEC) {
+    const int nvec = n / 8;
+    const long total = rows * nvec;
+    for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+      const long r = idx / nvec;
+      const int i = (idx % nvec) * 8;
+      float f[8];
+      ld8<T>(x + r * x_stride + i, f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) f[e] = op(f[e]);
+      st8<T>(out + r * n + i, f);
+    }
+  } else {
+    const long total = rows * n;
+    for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+      const long r = idx / n;
+      const int i = idx % n;
+      out[r * n + i] = ScalarOps<T>::from_f32(
+          op(ScalarOps<T>::to_f32(x[r * x_stride + i])));
+    }
+  }
+}
+
+template <typename Op>
+void launch_unary_rows(torch::Tensor &out, torch::Tensor &x, Op op,
+                       const char *name) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 2 && x.stride(1) == 1, name,
+              ": x must be [rows, n] with unit inner stride");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes() &&
+              out.scalar_type() == x.scalar_type());
+  const long rows = x.size(0);
+  const int n = x.size(1);
+  if (rows == 0 || n == 0) return;
+  const long esz = x.element_size();
+  const bool vec = n % 8 == 0 &&
+                   reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0 &&
+                   (x.stride(0) * esz) % 16 == 0;
+  const long work = vec ? rows * (n / 8) : rows * (long)n;
+  const int grid = (int)std::min<long>((work + 255) / 256, 65535);
+  auto stream = at::cuda::getCurrentCUDAStream();
+#define RUN(TT, V)                                                          \
+  hipLaunchKernelGGL((unary_rows_kernel<TT, Op, V>), dim3(grid), dim3(256), \
+                     0, stream, (TT *)out.data_ptr(),                       \
+                     (const TT *)x.data_ptr(), (long)x.stride(0), rows, n, op)
+  if (x.scalar_type() == at::kBFloat16) {
+    if (vec) RUN(__hip_bfloat16, true); else RUN(__hip_bfloat16, false);
+  } else if (x.scalar_type() == at::kFloat) {
+    if (vec) RUN(float, true); else RUN(float, false);
+  } else {
+    TORCH_CHECK(false, name, ": bf16 or fp32");
+  }
+#undef RUN
+  HIP_CHECK_KERNEL();
+}
+
+}  // namespace
+
+void xielu(torch::Tensor out, torch::Tensor x, double a_pos, double a_neg) {
+  launch_unary_rows(out, x, XieluOp{(float)a_pos, (float)a_neg}, "xielu");
+}
+
+void relu2(torch::Tensor out, torch::Tensor x) {
+  launch_unary_rows(out, x, Relu2Op{}, "relu2");
+}

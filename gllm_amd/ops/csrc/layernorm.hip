@@ -1,4 +1,4 @@
-// LayerNorm (weight + bias) over an fp32 residual stream, gfx950.
+// LayerNorm (weight + optional bias) over an fp32 residual stream, gfx950.
 //
 // The residual stream of a sandwich-norm decoder (norm before AND after
 // every sublayer) is kept in fp32 while the sublayers run in the model
@@ -6,6 +6,7 @@
 //
 //   layernorm_f32:      h = LN_pre(x)                       x fp32 -> h T
 //   residual_layernorm: x += LN_post(y); h = LN_pre(x)      y T, x fp32
+//                       with a gate: LN_post sees y * sigmoid(gate)
 //
 // One workgroup per token row; the row lives in LDS as fp32 between the
 // mean, variance (mean of squared deviations, two passes: no E[x^2] -
@@ -68,9 +69,9 @@ DEV_INLINE void ln_row(float *row, const T *__restrict__ w,
   const float inv = 1.0f / sqrtf(var + eps);
   if (vec) {
     for (int i = threadIdx.x * 8; i < width; i += LN_BLOCK * 8) {
-      float wf[8], bf[8];
+      float wf[8], bf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       ld8<T>(w + i, wf);
-      ld8<T>(b + i, bf);
+      if (b) ld8<T>(b + i, bf);
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         row[i + e] = (row[i + e] - mean) * inv * wf[e] + bf[e];
@@ -78,9 +79,27 @@ DEV_INLINE void ln_row(float *row, const T *__restrict__ w,
   } else {
     for (int i = threadIdx.x; i < width; i += LN_BLOCK)
       row[i] = (row[i] - mean) * inv * ScalarOps<T>::to_f32(w[i]) +
-               ScalarOps<T>::to_f32(b[i]);
+               (b ? ScalarOps<T>::to_f32(b[i]) : 0.f);
   }
   __syncthreads();
+}
+
+DEV_INLINE float sigmoid_f32(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// row *= sigmoid(gate row); same thread-to-element mapping as row_load
+template <typename T>
+DEV_INLINE void row_gate(float *row, const T *g, int width, bool vec) {
+  if (vec) {
+    for (int i = threadIdx.x * 8; i < width; i += LN_BLOCK * 8) {
+      float gf[8];
+      ld8<T>(g + i, gf);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) row[i + e] *= sigmoid_f32(gf[e]);
+    }
+  } else {
+    for (int i = threadIdx.x; i < width; i += LN_BLOCK)
+      row[i] *= sigmoid_f32(ScalarOps<T>::to_f32(g[i]));
+  }
 }
 
 template <typename T>
@@ -103,11 +122,13 @@ __global__ __launch_bounds__(LN_BLOCK) void residual_layernorm_kernel(
     float *__restrict__ x, const T *__restrict__ y, long y_stride,
     const T *__restrict__ w_post, const T *__restrict__ b_post,
     T *__restrict__ h, const T *__restrict__ w_pre,
-    const T *__restrict__ b_pre, float eps, int width, int vec) {
+    const T *__restrict__ b_pre, float eps, int width, int vec,
+    const T *__restrict__ gate, long gate_stride) {
   extern __shared__ float row[];
   __shared__ float red[LN_BLOCK / WAVE_SIZE];
   const long base = (long)blockIdx.x * width;
   row_load<T>(row, y + (long)blockIdx.x * y_stride, width, vec);
+  if (gate) row_gate<T>(row, gate + (long)blockIdx.x * gate_stride, width, vec);
   __syncthreads();
   ln_row<T>(row, w_post, b_post, eps, width, red, vec);
   if (vec) {
@@ -143,7 +164,8 @@ __global__ __launch_bounds__(LN_BLOCK) void residual_layernorm_wave_kernel(
     float *__restrict__ x, const T *__restrict__ y, long y_stride,
     const T *__restrict__ w_post, const T *__restrict__ b_post,
     T *__restrict__ h, const T *__restrict__ w_pre,
-    const T *__restrict__ b_pre, float eps, int width, long rows) {
+    const T *__restrict__ b_pre, float eps, int width, long rows,
+    const T *__restrict__ gate, long gate_stride) {
   const int lane = threadIdx.x & 63;
   const long row = (long)blockIdx.x * (LN_BLOCK / 64) + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -156,6 +178,12 @@ __global__ __launch_bounds__(LN_BLOCK) void residual_layernorm_wave_kernel(
     const int i = (c * 64 + lane) * 8;
     if (i < width) {
       ld8<T>(yr + i, r[c]);
+      if (gate) {
+        float gf[8];
+        ld8<T>(gate + row * gate_stride + i, gf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r[c][e] *= sigmoid_f32(gf[e]);
+      }
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) r[c][e] = 0.f;
@@ -181,9 +209,9 @@ __global__ __launch_bounds__(LN_BLOCK) void residual_layernorm_wave_kernel(
   for (int c = 0; c < NCH; ++c) {
     const int i = (c * 64 + lane) * 8;
     if (i < width) {
-      float wf[8], bf[8], xf[8];
+      float wf[8], bf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, xf[8];
       ld8<T>(w_post + i, wf);
-      ld8<T>(b_post + i, bf);
+      if (b_post) ld8<T>(b_post + i, bf);
       ld8<float>(x + base + i, xf);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -212,9 +240,9 @@ __global__ __launch_bounds__(LN_BLOCK) void residual_layernorm_wave_kernel(
   for (int c = 0; c < NCH; ++c) {
     const int i = (c * 64 + lane) * 8;
     if (i < width) {
-      float wf[8], bf[8], of[8];
+      float wf[8], bf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, of[8];
       ld8<T>(w_pre + i, wf);
-      ld8<T>(b_pre + i, bf);
+      if (b_pre) ld8<T>(b_pre + i, bf);
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         of[e] = (r[c][e] - mean) * inv * wf[e] + bf[e];
@@ -235,7 +263,7 @@ void check_vec(const torch::Tensor &t, int width, at::ScalarType st) {
 }  // namespace
 
 void layernorm_f32(torch::Tensor out, torch::Tensor x, torch::Tensor w,
-                   torch::Tensor b, double eps) {
+                   c10::optional<torch::Tensor> b, double eps) {
   TORCH_CHECK(x.scalar_type() == at::kFloat && x.is_contiguous());
   TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes());
   const int width = x.size(-1);
@@ -243,16 +271,20 @@ void layernorm_f32(torch::Tensor out, torch::Tensor x, torch::Tensor w,
   if (rows == 0) return;
   TORCH_CHECK(width > 0 && width * 4 <= 64 * 1024);
   check_vec(w, width, out.scalar_type());
-  check_vec(b, width, out.scalar_type());
+  const void *bp = nullptr;
+  if (b.has_value()) {
+    check_vec(*b, width, out.scalar_type());
+    bp = b->data_ptr();
+  }
   const int vec = (width % 8 == 0 && aligned16(x.data_ptr()) &&
                    aligned16(out.data_ptr()) && aligned16(w.data_ptr()) &&
-                   aligned16(b.data_ptr())) ? 1 : 0;
+                   aligned16(bp)) ? 1 : 0;
   auto stream = at::cuda::getCurrentCUDAStream();
 #define RUN(T)                                                             \
   hipLaunchKernelGGL((layernorm_f32_kernel<T>), dim3(rows), dim3(LN_BLOCK), \
                      width * sizeof(float), stream, (T *)out.data_ptr(),   \
                      x.data_ptr<float>(), (const T *)w.data_ptr(),         \
-                     (const T *)b.data_ptr(), (float)eps, width, vec)
+                     (const T *)bp, (float)eps, width, vec)
   if (out.scalar_type() == at::kBFloat16) RUN(__hip_bfloat16);
   else if (out.scalar_type() == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "layernorm_f32: bf16 or fp32 output");
@@ -261,10 +293,12 @@ void layernorm_f32(torch::Tensor out, torch::Tensor x, torch::Tensor w,
 }
 
 void residual_layernorm(torch::Tensor x, torch::Tensor y,
-                        torch::Tensor w_post, torch::Tensor b_post,
+                        torch::Tensor w_post,
+                        c10::optional<torch::Tensor> b_post,
                         c10::optional<torch::Tensor> h,
                         c10::optional<torch::Tensor> w_pre,
-                        c10::optional<torch::Tensor> b_pre, double eps) {
+                        c10::optional<torch::Tensor> b_pre, double eps,
+                        c10::optional<torch::Tensor> gate) {
   TORCH_CHECK(x.scalar_type() == at::kFloat && x.is_contiguous());
   const int width = x.size(-1);
   const long rows = x.numel() / std::max(width, 1);
@@ -274,24 +308,41 @@ void residual_layernorm(torch::Tensor x, torch::Tensor y,
               y.stride(1) == 1, "residual_layernorm: y must be [rows, width]");
   const auto st = y.scalar_type();
   check_vec(w_post, width, st);
-  check_vec(b_post, width, st);
+  const void *bpost = nullptr;
+  if (b_post.has_value()) {
+    check_vec(*b_post, width, st);
+    bpost = b_post->data_ptr();
+  }
   void *hp = nullptr;
   const void *wp = nullptr, *bp = nullptr;
   if (h.has_value()) {
-    TORCH_CHECK(w_pre.has_value() && b_pre.has_value());
+    TORCH_CHECK(w_pre.has_value());
     TORCH_CHECK(h->is_contiguous() && h->numel() == x.numel() &&
                 h->scalar_type() == st);
     check_vec(*w_pre, width, st);
-    check_vec(*b_pre, width, st);
     hp = h->data_ptr();
     wp = w_pre->data_ptr();
-    bp = b_pre->data_ptr();
+    if (b_pre.has_value()) {
+      check_vec(*b_pre, width, st);
+      bp = b_pre->data_ptr();
+    }
+  }
+  const void *gp = nullptr;
+  long gs = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->is_cuda() && gate->dim() == 2 &&
+                gate->size(0) == rows && gate->size(1) == width &&
+                gate->stride(1) == 1 && gate->scalar_type() == st,
+                "residual_layernorm: gate must be [rows, width]");
+    gp = gate->data_ptr();
+    gs = gate->stride(0);
   }
   const int vec =
       (width % 8 == 0 && aligned16(x.data_ptr()) && aligned16(y.data_ptr()) &&
        (y.stride(0) * y.element_size()) % 16 == 0 &&
-       aligned16(w_post.data_ptr()) && aligned16(b_post.data_ptr()) &&
-       aligned16(hp) && aligned16(wp) && aligned16(bp)) ? 1 : 0;
+       aligned16(w_post.data_ptr()) && aligned16(bpost) &&
+       aligned16(hp) && aligned16(wp) && aligned16(bp) && aligned16(gp) &&
+       (gs * y.element_size()) % 16 == 0) ? 1 : 0;
   auto stream = at::cuda::getCurrentCUDAStream();
   if (vec && width <= 8192) {
     const int nch = width <= 512 ? 1 : width <= 1024 ? 2 : width <= 2048 ? 4
@@ -302,8 +353,9 @@ void residual_layernorm(torch::Tensor x, torch::Tensor y,
                      dim3(LN_BLOCK), 0, stream, x.data_ptr<float>(),        \
                      (const T *)y.data_ptr(), (long)y.stride(0),            \
                      (const T *)w_post.data_ptr(),                          \
-                     (const T *)b_post.data_ptr(), (T *)hp, (const T *)wp,  \
-                     (const T *)bp, (float)eps, width, rows)
+                     (const T *)bpost, (T *)hp, (const T *)wp,              \
+                     (const T *)bp, (float)eps, width, rows,                \
+                     (const T *)gp, gs)
 #define RUNW_N(T)                                                           \
   switch (nch) {                                                            \
     case 1: RUNW(T, 1); break;                                              \
@@ -325,8 +377,9 @@ void residual_layernorm(torch::Tensor x, torch::Tensor y,
                      dim3(LN_BLOCK), width * sizeof(float), stream,         \
                      x.data_ptr<float>(), (const T *)y.data_ptr(),          \
                      (long)y.stride(0), (const T *)w_post.data_ptr(),       \
-                     (const T *)b_post.data_ptr(), (T *)hp, (const T *)wp,  \
-                     (const T *)bp, (float)eps, width, vec)
+                     (const T *)bpost, (T *)hp, (const T *)wp,              \
+                     (const T *)bp, (float)eps, width, vec,                 \
+                     (const T *)gp, gs)
   if (st == at::kBFloat16) RUN(__hip_bfloat16);
   else if (st == at::kFloat) RUN(float);
   else TORCH_CHECK(false, "residual_layernorm: bf16 or fp32 sublayer output");

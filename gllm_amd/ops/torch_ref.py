@@ -260,43 +260,66 @@ def apply_repetition_penalty(logits: torch.Tensor, token_ids_per_row,
 # fp32-residual layer norm / windowed sink attention (CPU path + kernel
 # oracle for ops.layernorm_f32, residual_layernorm, qk_norm_rope_store,
 # window_attention)
-def layernorm_f32(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor,
-                  eps: float, dtype) -> torch.Tensor:
-    """LayerNorm of an fp32 row with weight and bias, output in ``dtype``."""
+def layernorm_f32(x: torch.Tensor, w: torch.Tensor, b, eps: float,
+                  dtype) -> torch.Tensor:
+    """LayerNorm of an fp32 row with weight and optional bias (``b``
+    None: weight only), output in ``dtype``."""
     xf = x.float()
     mu = xf.mean(-1, keepdim=True)
     d = xf - mu
     var = (d * d).mean(-1, keepdim=True)
-    return (d * torch.rsqrt(var + eps) * w.float() + b.float()).to(dtype)
+    out = d * torch.rsqrt(var + eps) * w.float()
+    if b is not None:
+        out = out + b.float()
+    return out.to(dtype)
 
 
 def residual_layernorm(x: torch.Tensor, y: torch.Tensor, w_post, b_post,
-                       eps: float, pre=None):
+                       eps: float, pre=None, gate=None):
     """x (fp32, in place) += LN(y); returns LN_pre(x) when ``pre`` is a
-    (weight, bias) pair."""
-    x.add_(layernorm_f32(y, w_post, b_post, eps, torch.float32))
+    (weight, bias) pair. ``gate`` (logits, same shape as y): the norm
+    sees y * sigmoid(gate)."""
+    yf = y.float()
+    if gate is not None:
+        yf = yf * torch.sigmoid(gate.float())
+    x.add_(layernorm_f32(yf, w_post, b_post, eps, torch.float32))
     if pre is None:
         return None
     return layernorm_f32(x, pre[0], pre[1], eps, y.dtype)
 
 
 def qk_norm_rope_store(q, k, v, q_w, k_w, positions, slot_mapping, freqs,
-                       mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps):
-    """Per-head RMS norm (plain weight) + interleaved-pair rotary on q
-    (in place) and k; k, v land in the paged cache rows ``slot_mapping``.
-    ``k`` None: a layer that reads another layer's cache."""
+                       mag, rot_dims, k_cache, v_cache, H, G, D, Dv, eps,
+                       half_layout=False, norm_last=False):
+    """Per-head RMS norm (plain weight, or none when the weight is None)
+    + rotary on q (in place) and k; k, v land in the paged cache rows
+    ``slot_mapping``. ``k`` None: a layer that reads another layer's
+    cache. ``half_layout``: dimension i pairs with i + rot_dims/2
+    instead of (2i, 2i+1); ``norm_last``: rotate first, then norm."""
     T = q.shape[0]
     ang = positions[:T].double()[:, None] * freqs.double()[None, :rot_dims // 2]
     cos = (torch.cos(ang).float() * mag)[:, None, :]
     sin = (torch.sin(ang).float() * mag)[:, None, :]
+    half = rot_dims // 2
 
-    def prep(x, w, heads):
-        xf = x.float().reshape(T, heads, D)
-        xf = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps) \
-            * w.float()
+    def norm(xf, w):
+        xf = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
+        return xf if w is None else xf * w.float()
+
+    def rotate(xf):
+        if half_layout:
+            a, b = xf[..., :half], xf[..., half:rot_dims]
+            return torch.cat([a * cos - b * sin, b * cos + a * sin,
+                              xf[..., rot_dims:]], dim=-1)
         a, b = xf[..., 0:rot_dims:2], xf[..., 1:rot_dims:2]
         rot = torch.stack([a * cos - b * sin, b * cos + a * sin], dim=-1)
         return torch.cat([rot.flatten(-2), xf[..., rot_dims:]], dim=-1)
+
+    def prep(x, w, heads):
+        xf = x.float().reshape(T, heads, D)
+        if norm_last:
+            return norm(rotate(xf), w)
+        return rotate(norm(xf, w))
 
     q.copy_(prep(q, q_w, H).reshape(T, H * D).to(q.dtype))
     if k is None:
@@ -349,6 +372,59 @@ def window_attention(q, gate, k_cache, v_cache, block_table, seq_lens,
     if gate is not None:
         out = out * torch.sigmoid(gate.float())
     return out.to(q.dtype)
+
+
+def talking_attention(q, k_cache, v_cache, block_table, seq_lens,
+                      query_start_loc, scale, talk, sink):
+    """Ragged paged causal attention whose per-head score planes are
+    mixed across heads before the softmax: s'_h = sum_g talk[h, g] s_g
+    with s_g = scale * q_g . k. ``sink`` [H] (or None) adds exp(sink_h)
+    to head h's softmax denominator. Scores and weights are fp32."""
+    page, G, D = k_cache.shape[1:]
+    Dv = v_cache.shape[3]
+    T = q.shape[0]
+    H = q.shape[1] // D
+    out = torch.zeros(T, H, Dv, dtype=torch.float32)
+    qsl = query_start_loc.tolist()
+    lens = seq_lens.tolist()
+    qf = q.float().reshape(T, H, D)
+    mix = talk.float()
+    for b in range(len(lens)):
+        s, e, L = qsl[b], qsl[b + 1], lens[b]
+        if e == s:
+            continue
+        pages = block_table[b, :-(-L // page)].long()
+        kk = k_cache[pages].reshape(-1, G, D)[:L].float()
+        vv = v_cache[pages].reshape(-1, G, Dv)[:L].float()
+        pos_i = torch.arange(L - (e - s), L)[:, None]
+        see = torch.arange(L)[None, :] <= pos_i
+        kk = kk.repeat_interleave(H // G, dim=1)
+        vv = vv.repeat_interleave(H // G, dim=1)
+        sc = torch.einsum("ihd,jhd->hij", qf[s:e], kk) * scale
+        sc = torch.einsum("hg,gij->hij", mix, sc)
+        sc = sc.masked_fill(~see[None], float("-inf"))
+        m = sc.amax(-1, keepdim=True)
+        if sink is not None:
+            sk = sink.float().view(H, 1, 1)
+            m = torch.maximum(m, sk)
+        p = torch.exp(sc - m)
+        den = p.sum(-1, keepdim=True)
+        if sink is not None:
+            den = den + torch.exp(sk - m)
+        out[s:e] = torch.einsum("hij,jhd->ihd", p / den, vv)
+    return out.reshape(T, H * Dv).to(q.dtype)
+
+
+def xielu(x: torch.Tensor, a_pos: float, a_neg: float) -> torch.Tensor:
+    """z > 0: a_pos z^2 + z/2; z <= 0: a_neg (exp(z) - 1 - z) + z/2."""
+    z = x.float()
+    neg = a_neg * (torch.expm1(z.clamp(max=0.0)) - z) + 0.5 * z
+    return torch.where(z > 0, a_pos * z * z + 0.5 * z, neg).to(x.dtype)
+
+
+def relu2(x: torch.Tensor) -> torch.Tensor:
+    r = torch.relu(x.float())
+    return (r * r).to(x.dtype)
 
 
 def topk_then_softmax(logits: torch.Tensor, topk: int):

@@ -33,6 +33,7 @@ HIP_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
 CXX_FLAGS = ["-O3", "-std=c++17"]
 
 SEQ_SOURCES = ["bindings_seq.cpp", "layernorm.hip", "attention_window.hip",
+               "attention_talking.hip",
                "attention_prefill.hip", "attention_decode.hip",
                "delta_rule.hip", "moe.hip", "elementwise.hip",
                "skinny_gemm.hip"]
