@@ -238,12 +238,55 @@ def hybrid_gdn_config(sz, vocab=32000):
             "vocab_size": vocab}
 
 
+def gukirax_config(sz, vocab=32000):
+    """Attention-only looped stack: 6 layers, the first two run twice
+    (8 layer runs), MoE with a shared expert in every layer."""
+    H, G, D = sz["attn"]
+    mlp = {"kind": "moe", "expert": {"ff": sz["ff"]},
+           "router": {"experts": sz["experts"], "top": sz["top"]},
+           "shared": {"ff": sz["ff"]}}
+    layer = {"type": "attention", "mlp": mlp, "mixer": {
+        "heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5,
+        "rot": {"dims": D // 4, "base": 1000000.0}}}
+    n = sz["layers"] - 2
+    return {"architecture": "Gukirax", "layers": [layer] * n,
+            "loop": {"start": 0, "stop": 2, "times": 2},
+            "logit_scale": 1.0, "logit_softcap": 30.0,
+            "norm": {"eps": 1e-5}, "vocab": vocab, "vocab_size": vocab,
+            "width": sz["width"]}
+
+
+def sudevik_attention_config(sz, vocab=32000):
+    """The closest existing stack: Sudevik with attention mixers only
+    (sink attention, sigmoid gate, fp32 LayerNorm stream, MoE), as many
+    layers as the Gukirax stack has layer runs."""
+    H, G, D = sz["attn"]
+    mlp = {"kind": "moe", "expert": {"ff": sz["ff"]},
+           "router": {"experts": sz["experts"], "top": sz["top"]}}
+    layer = {"type": "attention", "mlp": mlp, "mixer": {
+        "heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5,
+        "rot": {"dims": D // 4, "base": 1000000.0}}}
+    return {"architecture": "Sudevik", "layers": [layer] * sz["layers"],
+            "norm": {"eps": 1e-5}, "vocab": vocab, "vocab_size": vocab,
+            "width": sz["width"]}
+
+
+COMPARE_PAIRS = {
+    "sudevik": (("sudevik", sudevik_config),
+                ("hybrid-gdn", hybrid_gdn_config)),
+    "gukirax": (("gukirax", gukirax_config),
+                ("sudevik-attn", sudevik_attention_config)),
+}
+
+
 # the same two 8-layer stacks as --model choices of the flagship workload
 # (scheduler policies, overlap engine, hipGraph decode buckets)
 MODELS["sudevik-w2048"] = ("Sudevik-w2048-8L",
                            sudevik_config(COMPARE_SIZES["w2048"]))
 MODELS["hybrid-gdn-w2048"] = ("hybrid-GDN-w2048-8L",
                               hybrid_gdn_config(COMPARE_SIZES["w2048"]))
+MODELS["gukirax-w2048"] = ("Gukirax-w2048-8runs",
+                           gukirax_config(COMPARE_SIZES["w2048"]))
 
 
 def mixer_compare(args):
@@ -255,8 +298,8 @@ def mixer_compare(args):
     P = args.prompt_len
     for size_name in args.compare_sizes.split(","):
         sz = COMPARE_SIZES[size_name]
-        for fam, cfg_json in (("sudevik", sudevik_config(sz)),
-                              ("hybrid-gdn", hybrid_gdn_config(sz))):
+        for fam, make_cfg in COMPARE_PAIRS[args.compare_pair]:
+            cfg_json = make_cfg(sz)
             cfg = EngineConfig(
                 model=write_model_dir(cfg_json), load_format="dummy",
                 dtype="bfloat16" if use_gpu else "float32", device=device,
@@ -373,6 +416,12 @@ def main():
                          "the hybrid-GDN family at equal layer sizes, "
                          "prefill and decode tokens/s (one JSON line per "
                          "case)")
+    ap.add_argument("--compare-pair", type=str, default="sudevik",
+                    choices=sorted(COMPARE_PAIRS),
+                    help="with --mixer-compare: 'sudevik' = Sudevik vs "
+                         "hybrid-GDN; 'gukirax' = Gukirax (looped "
+                         "talking-heads attention) vs an attention-only "
+                         "Sudevik stack of as many layer runs")
     ap.add_argument("--compare-sizes", type=str, default="w2048,w1024")
     ap.add_argument("--compare-decode", type=str, default="1,32,128")
     ap.add_argument("--compare-prefill-batch", type=int, default=4)

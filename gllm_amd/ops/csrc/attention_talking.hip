@@ -17,11 +17,11 @@
 //       -> LDS, mix + online softmax (one wave per head), P.V with the
 //       accumulators in registers. Decode-only batches split the keys
 //       over several workgroups (partials + talking_merge_kernel).
-//   talking_mfma_kernel        bf16, D == Dv a multiple of 32, batches
-//       with prompt portions: 32 queries of one sequence per workgroup,
-//       K/V tiles of 32 keys staged through LDS, S^T = K Q^T and
-//       O^T = V^T P^T on 32x32x8 MFMA; the raw score planes of all heads
-//       pass through LDS for the fp32 mix.
+//   talking_mfma_kernel        bf16, D == Dv in {32, 64, 96, 128}, up to
+//       16 heads, batches with prompt portions: 16 queries of one
+//       sequence per workgroup, K/V tiles of 32 keys staged through LDS,
+//       Q K^T and P V on 16x16x32 MFMA; the raw score planes of all
+//       heads pass through LDS for the fp32 mix.
 
 #include <torch/extension.h>
 #include <ATen/cuda/CUDAContext.h>
@@ -343,7 +343,278 @@ void talking_attention(torch::Tensor out, torch::Tensor q,
   }
 }
 
-// the MFMA tile form is added below this line
+// ------------------------------------------------------------------
+// MFMA tile form (bf16). One workgroup = 16 queries of one sequence x
+// all H heads; 4 waves, wave w owns heads w, w+4, ... (HPW per wave).
+// Per 32-key tile:
+//   stage K (all kv heads) -> LDS
+//   S_h = Q_h K^T on 16x16x32 MFMA, scaled, -> sraw[h] (fp32, LDS)
+//   stage V over K; meanwhile mix: s'_h = sum_g talk[h,g] sraw[g]
+//   (lane = query row x 8 keys, 16 B LDS reads), causal mask, online
+//   softmax in fp32, P_h -> pbuf[h] (bf16), rescale factors -> LDS
+//   O_h += P_h V on MFMA (B fragments gathered from the linear V tile)
+// Softmax weights are fp32 until they become the matrix core's left
+// operand (bf16, fp32 accumulation); scores, mix, max/sum and the sink
+// never leave fp32.
+typedef __attribute__((ext_vector_type(8))) __bf16 tk_bf8;
+typedef __attribute__((ext_vector_type(4))) float tk_f4;
+
+namespace {
+
+constexpr int MQ = 16;   // queries per workgroup
+constexpr int MK = 32;   // keys per tile
+constexpr int MWAVES = 4;
+constexpr int SR = 36;   // sraw row stride (floats), 16 B aligned rows
+constexpr int PR = 40;   // pbuf row stride (bf16), 16 B aligned rows
+
+template <int D, int HPW>
+__global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
+    __hip_bfloat16 *__restrict__ out, const __hip_bfloat16 *__restrict__ q,
+    long q_stride, const __hip_bfloat16 *__restrict__ k_cache,
+    const __hip_bfloat16 *__restrict__ v_cache,
+    const int *__restrict__ block_table, int bt_stride,
+    const int *__restrict__ seq_lens, const int *__restrict__ qsl, int H,
+    int G, int page, float scale, const float *__restrict__ talk,
+    const float *__restrict__ sink) {
+  constexpr int KT = D / 32, NT = D / 16, KS = D + 8, CPR = D / 8;
+  extern __shared__ __attribute__((aligned(16))) char tk_lds[];
+  __hip_bfloat16 *kvbuf = reinterpret_cast<__hip_bfloat16 *>(tk_lds);
+  float *sraw = reinterpret_cast<float *>(tk_lds + (size_t)G * MK * KS * 2);
+  __hip_bfloat16 *pbuf =
+      reinterpret_cast<__hip_bfloat16 *>(sraw + H * MQ * SR);
+  float *alpha_s = reinterpret_cast<float *>(pbuf + H * MQ * PR);
+  float *tks = alpha_s + H * MQ;
+
+  const int tile = blockIdx.x, b = blockIdx.y;
+  const int q_start = qsl[b];
+  const int q_len = qsl[b + 1] - q_start;
+  if (tile * MQ >= q_len) return;
+  const int seq_len = seq_lens[b];
+  const int past = seq_len - q_len;
+  const int rep = H / G;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, lhi = lane >> 4;
+  const int mi = lane >> 2, mc = lane & 3;   // mix layout: row, key octet
+  const int *bt = block_table + (long)b * bt_stride;
+
+  for (int d = tid; d < H * H; d += MWAVES * 64) tks[d] = talk[d];
+
+  float m_run[HPW], l_run[HPW];
+  tk_f4 o_acc[HPW][NT];
+#pragma unroll
+  for (int hs = 0; hs < HPW; ++hs) {
+    m_run[hs] = -INFINITY;
+    l_run[hs] = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) o_acc[hs][nt] = tk_f4{0, 0, 0, 0};
+  }
+  const int qrow_a = tile * MQ + l16;          // A-fragment row
+  const bool qrow_a_ok = qrow_a < q_len;
+  const __hip_bfloat16 *qa =
+      q + (long)(q_start + (qrow_a_ok ? qrow_a : 0)) * q_stride + lhi * 8;
+  const int qrow_m = tile * MQ + mi;
+  const int qpos_m = past + qrow_m;
+  const bool qrow_m_ok = qrow_m < q_len;
+  const int kv_max = min(seq_len, past + min(q_len, (tile + 1) * MQ));
+
+  auto stage = [&](const __hip_bfloat16 *__restrict__ src, int kv0) {
+    const int per_key = G * CPR;
+    for (int c = tid; c < MK * per_key; c += MWAVES * 64) {
+      const int key = c / per_key, rem = c - key * per_key;
+      const int g = rem / CPR, dc = rem - g * CPR;
+      const int tok = min(kv0 + key, seq_len - 1);
+      const long row = (long)bt[tok / page] * page + tok % page;
+      *reinterpret_cast<shortx8 *>(&kvbuf[(g * MK + key) * KS + dc * 8]) =
+          *reinterpret_cast<const shortx8 *>(src + (row * G + g) * D + dc * 8);
+    }
+  };
+
+  for (int kv0 = 0; kv0 < kv_max; kv0 += MK) {
+    stage(k_cache, kv0);
+    __syncthreads();
+    // ---- raw scores of this wave's heads ----
+#pragma unroll
+    for (int hs = 0; hs < HPW; ++hs) {
+      const int h = wave + hs * MWAVES;
+      if (h < H) {
+        const int g = h / rep;
+        tk_f4 s0 = tk_f4{0, 0, 0, 0}, s1 = tk_f4{0, 0, 0, 0};
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+          tk_bf8 a = tk_bf8{0, 0, 0, 0, 0, 0, 0, 0};
+          if (qrow_a_ok)
+            a = *reinterpret_cast<const tk_bf8 *>(qa + h * D + kt * 32);
+          const tk_bf8 b0 = *reinterpret_cast<const tk_bf8 *>(
+              &kvbuf[(g * MK + l16) * KS + kt * 32 + lhi * 8]);
+          const tk_bf8 b1 = *reinterpret_cast<const tk_bf8 *>(
+              &kvbuf[(g * MK + 16 + l16) * KS + kt * 32 + lhi * 8]);
+          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b0, s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b1, s1, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float *row = sraw + (h * MQ + lhi * 4 + r) * SR;
+          row[l16] = s0[r] * scale;
+          row[16 + l16] = s1[r] * scale;
+        }
+      }
+    }
+    __syncthreads();
+    stage(v_cache, kv0);   // K is done with; V lands while the heads talk
+    // ---- mix + online softmax ----
+#pragma unroll
+    for (int hs = 0; hs < HPW; ++hs) {
+      const int h = wave + hs * MWAVES;
+      if (h < H) {
+        float sv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sv[e] = 0.f;
+        for (int g2 = 0; g2 < H; ++g2) {
+          const float t = tks[h * H + g2];
+          const float *row = sraw + (g2 * MQ + mi) * SR + mc * 8;
+          const floatx4 a0 = *reinterpret_cast<const floatx4 *>(row);
+          const floatx4 a1 = *reinterpret_cast<const floatx4 *>(row + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            sv[e] += t * a0[e];
+            sv[4 + e] += t * a1[e];
+          }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int kvp = kv0 + mc * 8 + e;
+          if (!qrow_m_ok || kvp > qpos_m || kvp >= seq_len) sv[e] = -INFINITY;
+          mx = fmaxf(mx, sv[e]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+        const float m_old = m_run[hs];
+        const float m_new = fmaxf(m_old, mx);
+        float pv[8], psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pv[e] = sv[e] == -INFINITY ? 0.f : expf(sv[e] - m_new);
+          psum += pv[e];
+        }
+        psum += __shfl_xor(psum, 1, 64);
+        psum += __shfl_xor(psum, 2, 64);
+        const float alpha = m_old == -INFINITY ? 0.f : expf(m_old - m_new);
+        l_run[hs] = l_run[hs] * alpha + psum;
+        m_run[hs] = m_new;
+        if (mc == 0) alpha_s[h * MQ + mi] = alpha;
+        *reinterpret_cast<shortx8 *>(&pbuf[(h * MQ + mi) * PR + mc * 8]) =
+            pack8<__hip_bfloat16>(pv);
+      }
+    }
+    __syncthreads();
+    // ---- O += P V ----
+#pragma unroll
+    for (int hs = 0; hs < HPW; ++hs) {
+      const int h = wave + hs * MWAVES;
+      if (h < H) {
+        const int g = h / rep;
+        float a4[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) a4[r] = alpha_s[h * MQ + lhi * 4 + r];
+        const tk_bf8 pf = *reinterpret_cast<const tk_bf8 *>(
+            &pbuf[(h * MQ + l16) * PR + lhi * 8]);
+        const __hip_bfloat16 *vt = kvbuf + (g * MK + lhi * 8) * KS + l16;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          tk_bf8 vf;
+          __hip_bfloat16 *ve = reinterpret_cast<__hip_bfloat16 *>(&vf);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) ve[j] = vt[j * KS + nt * 16];
+          tk_f4 acc = o_acc[hs][nt];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[r] *= a4[r];
+          o_acc[hs][nt] =
+              __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, acc, 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: sink joins the denominator, rows leave as bf16 ----
+#pragma unroll
+  for (int hs = 0; hs < HPW; ++hs) {
+    const int h = wave + hs * MWAVES;
+    if (h < H && mc == 0) {
+      float m = m_run[hs], l = l_run[hs], w = 1.f;
+      if (sink != nullptr) {
+        const float sk = sink[h];
+        const float M = fmaxf(m, sk);
+        w = m == -INFINITY ? 0.f : expf(m - M);
+        l = l * w + expf(sk - M);
+      }
+      alpha_s[h * MQ + mi] = l > 0.f ? w / l : 0.f;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int hs = 0; hs < HPW; ++hs) {
+    const int h = wave + hs * MWAVES;
+    if (h < H) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int qrow = tile * MQ + lhi * 4 + r;
+        if (qrow >= q_len) continue;
+        const float f = alpha_s[h * MQ + lhi * 4 + r];
+        __hip_bfloat16 *op = out + ((long)(q_start + qrow) * H + h) * D + l16;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          op[nt * 16] = __float2bfloat16(o_acc[hs][nt][r] * f);
+      }
+    }
+  }
+}
+
+template <int D, int HPW>
+bool launch_talking_mfma(torch::Tensor &out, torch::Tensor &q,
+                         torch::Tensor &k_cache, torch::Tensor &v_cache,
+                         torch::Tensor &block_table, torch::Tensor &seq_lens,
+                         torch::Tensor &query_start_loc, double scale,
+                         torch::Tensor &talk, const float *sink,
+                         long max_query_len, int H, int G, int page) {
+  const size_t lds = (size_t)G * MK * (D + 8) * 2 + (size_t)H * MQ * SR * 4 +
+                     (size_t)H * MQ * PR * 2 + (size_t)H * MQ * 4 +
+                     (size_t)H * H * 4;
+  if (lds > 160 * 1024) return false;
+  auto kern = talking_mfma_kernel<D, HPW>;
+  if (lds > 48 * 1024) {
+    static size_t granted = 0;   // per instantiation
+    if (lds > granted) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+      }
+      granted = lds;
+    }
+  }
+  const int B = seq_lens.numel();
+  const int q_tiles = (int)((max_query_len + MQ - 1) / MQ);
+  auto stream = at::cuda::getCurrentCUDAStream();
+  hipLaunchKernelGGL(kern, dim3(q_tiles, B), dim3(MWAVES * 64), lds, stream,
+                     (__hip_bfloat16 *)out.data_ptr(),
+                     (const __hip_bfloat16 *)q.data_ptr(), (long)q.stride(0),
+                     (const __hip_bfloat16 *)k_cache.data_ptr(),
+                     (const __hip_bfloat16 *)v_cache.data_ptr(),
+                     block_table.data_ptr<int>(), (int)block_table.stride(0),
+                     seq_lens.data_ptr<int>(),
+                     query_start_loc.data_ptr<int>(), H, G, page,
+                     (float)scale, talk.data_ptr<float>(), sink);
+  HIP_CHECK_KERNEL();
+  return true;
+}
+
+}  // namespace
+
+// false = this geometry has no MFMA instantiation (the caller runs the
+// generic kernel)
 bool talking_attention_mfma(torch::Tensor &out, torch::Tensor &q,
                             torch::Tensor &k_cache, torch::Tensor &v_cache,
                             torch::Tensor &block_table,
@@ -351,5 +622,29 @@ bool talking_attention_mfma(torch::Tensor &out, torch::Tensor &q,
                             torch::Tensor &query_start_loc, double scale,
                             torch::Tensor &talk, const float *sink,
                             long max_query_len) {
+  const int page = k_cache.size(1), G = k_cache.size(2), D = k_cache.size(3);
+  const int H = q.size(1) / D;
+  if (v_cache.size(3) != D || H > 4 * MWAVES) return false;
+  // 16 B fragment loads straight from q rows
+  if (reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 != 0 ||
+      (q.stride(0) * 2) % 16 != 0)
+    return false;
+  const int hpw = H <= MWAVES ? 1 : H <= 2 * MWAVES ? 2 : 4;
+#define GO(DV, HP)                                                          \
+  return launch_talking_mfma<DV, HP>(out, q, k_cache, v_cache, block_table, \
+                                     seq_lens, query_start_loc, scale,      \
+                                     talk, sink, max_query_len, H, G, page)
+#define GO_D(DV)                                                            \
+  if (D == DV) {                                                            \
+    if (hpw == 1) GO(DV, 1);                                                \
+    if (hpw == 2) GO(DV, 2);                                                \
+    GO(DV, 4);                                                              \
+  }
+  GO_D(32)
+  GO_D(64)
+  GO_D(96)
+  GO_D(128)
+#undef GO_D
+#undef GO
   return false;
 }
