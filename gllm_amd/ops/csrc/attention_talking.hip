@@ -195,29 +195,40 @@ __global__ __launch_bounds__(TK_BLOCK) void talking_attention_kernel(
   }
 }
 
-// grid (tokens): combine the key splits of one query, sink included
+// grid (tokens, heads): combine the key splits of one (query, head),
+// sink included; the first ``splits`` threads form the split weights
+constexpr int MERGE_MAX_SPLITS = 64;
+
 template <typename T>
-__global__ __launch_bounds__(TK_BLOCK) void talking_merge_kernel(
+__global__ __launch_bounds__(128) void talking_merge_kernel(
     T *__restrict__ out, const float *__restrict__ part_acc,
     const float *__restrict__ part_ml, const float *__restrict__ sink, int H,
     int Dv, int splits) {
-  const int t = blockIdx.x;
-  for (int o = threadIdx.x; o < H * Dv; o += TK_BLOCK) {
-    const int h = o / Dv;
-    float M = sink != nullptr ? sink[h] : -INFINITY;
-    for (int s = 0; s < splits; ++s)
-      M = fmaxf(M, part_ml[(((long)t * splits + s) * H + h) * 2]);
-    float l = sink != nullptr ? expf(sink[h] - M) : 0.f;
-    float a = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const long pb = (long)t * splits + s;
-      const float m = part_ml[(pb * H + h) * 2];
-      if (m == -INFINITY) continue;     // a split with no keys
-      const float w = expf(m - M);
-      l += part_ml[(pb * H + h) * 2 + 1] * w;
-      a += part_acc[pb * H * Dv + o] * w;
+  __shared__ float wgt[MERGE_MAX_SPLITS];
+  __shared__ float inv_l;
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x;
+  if (tid < 64) {
+    float m = -INFINITY, l = 0.f;
+    if (tid < splits) {
+      const long pb = ((long)t * splits + tid) * H + h;
+      m = part_ml[pb * 2];
+      l = part_ml[pb * 2 + 1];
     }
-    out[(long)t * H * Dv + o] = ScalarOps<T>::from_f32(a / l);
+    float M = wave_reduce_max(m);
+    if (sink != nullptr) M = fmaxf(M, sink[h]);
+    const float w = m == -INFINITY ? 0.f : expf(m - M);
+    if (tid < splits) wgt[tid] = w;
+    float lsum = wave_reduce_sum(l * w);
+    if (sink != nullptr) lsum += expf(sink[h] - M);
+    if (tid == 0) inv_l = lsum > 0.f ? 1.0f / lsum : 0.f;
+  }
+  __syncthreads();
+  for (int d = tid; d < Dv; d += 128) {
+    float a = 0.f;
+    for (int s = 0; s < splits; ++s)
+      a += part_acc[(((long)t * splits + s) * H + h) * Dv + d] * wgt[s];
+    out[((long)t * H + h) * Dv + d] = ScalarOps<T>::from_f32(a * inv_l);
   }
 }
 
@@ -234,6 +245,15 @@ bool talking_attention_mfma(torch::Tensor &out, torch::Tensor &q,
                             torch::Tensor &query_start_loc, double scale,
                             torch::Tensor &talk, const float *sink,
                             long max_query_len);
+
+bool talking_attention_decode_mfma(torch::Tensor &out, torch::Tensor &q,
+                                   torch::Tensor &k_cache,
+                                   torch::Tensor &v_cache,
+                                   torch::Tensor &block_table,
+                                   torch::Tensor &seq_lens, double scale,
+                                   torch::Tensor &talk, const float *sink,
+                                   int splits, float *part_acc,
+                                   float *part_ml);
 
 void talking_attention(torch::Tensor out, torch::Tensor q,
                        torch::Tensor k_cache, torch::Tensor v_cache,
@@ -297,13 +317,35 @@ void talking_attention(torch::Tensor out, torch::Tensor q,
     paccp = pacc.data_ptr<float>();
     pmlp = pml.data_ptr<float>();
   }
+  auto stream = at::cuda::getCurrentCUDAStream();
+  auto merge = [&]() {
+    if (splits == 1) return;
+    if (st == at::kBFloat16)
+      hipLaunchKernelGGL((talking_merge_kernel<__hip_bfloat16>), dim3(T, H),
+                         dim3(128), 0, stream,
+                         (__hip_bfloat16 *)out.data_ptr(), paccp, pmlp, sp, H,
+                         Dv, splits);
+    else
+      hipLaunchKernelGGL((talking_merge_kernel<float>), dim3(T, H),
+                         dim3(128), 0, stream, (float *)out.data_ptr(),
+                         paccp, pmlp, sp, H, Dv, splits);
+    HIP_CHECK_KERNEL();
+  };
+  // bf16 decode-only batch: one token per sequence, the heads of a GQA
+  // group ride the MFMA rows
+  if (st == at::kBFloat16 && max_query_len == 1 && T == B &&
+      talking_attention_decode_mfma(out, q, k_cache, v_cache, block_table,
+                                    seq_lens, scale, talk, sp, splits, paccp,
+                                    pmlp)) {
+    merge();
+    return;
+  }
   const int HD = (H * D + 3) & ~3, HH = (H * H + 3) & ~3;
   const int nf = (HD + HH + 2 * H * TK_KEYS + 3 * H + 1) & ~1;
   const size_t lds = (size_t)nf * sizeof(float) + TK_KEYS * sizeof(long);
   TORCH_CHECK(lds <= 64 * 1024, "talking_attention: heads * dim too large");
   int nacc = 1;
   while (nacc * TK_BLOCK < H * Dv) nacc *= 2;
-  auto stream = at::cuda::getCurrentCUDAStream();
 #define RUN(TT, N)                                                           \
   hipLaunchKernelGGL((talking_attention_kernel<TT, N>), dim3(T, splits),     \
                      dim3(TK_BLOCK), lds, stream, (TT *)out.data_ptr(),      \
@@ -329,18 +371,7 @@ void talking_attention(torch::Tensor out, torch::Tensor q,
 #undef RUN_N
 #undef RUN
   HIP_CHECK_KERNEL();
-  if (splits > 1) {
-    if (st == at::kBFloat16)
-      hipLaunchKernelGGL((talking_merge_kernel<__hip_bfloat16>), dim3(T),
-                         dim3(TK_BLOCK), 0, stream,
-                         (__hip_bfloat16 *)out.data_ptr(), paccp, pmlp, sp, H,
-                         Dv, splits);
-    else
-      hipLaunchKernelGGL((talking_merge_kernel<float>), dim3(T),
-                         dim3(TK_BLOCK), 0, stream, (float *)out.data_ptr(),
-                         paccp, pmlp, sp, H, Dv, splits);
-    HIP_CHECK_KERNEL();
-  }
+  merge();
 }
 
 // ------------------------------------------------------------------
@@ -366,6 +397,41 @@ constexpr int MK = 32;   // keys per tile
 constexpr int MWAVES = 4;
 constexpr int SR = 36;   // sraw row stride (floats), 16 B aligned rows
 constexpr int PR = 40;   // pbuf row stride (bf16), 16 B aligned rows
+
+// One K or V tile [G][MK keys][D] from the paged cache into LDS rows of
+// KS elements; 16 B chunks, loads issued four at a time before their
+// stores so the global latency is paid once per batch.
+template <int D>
+DEV_INLINE void stage_tile(__hip_bfloat16 *__restrict__ kvbuf,
+                           const __hip_bfloat16 *__restrict__ src,
+                           const int *__restrict__ bt, int page, int G,
+                           int kv0, int last_tok, int keys, int key_stride,
+                           int tid, int nthreads) {
+  constexpr int CPR = D / 8, KS = D + 8, U = 4;
+  const int per_key = G * CPR;
+  const int total = keys * per_key;
+  for (int c0 = tid; c0 < total; c0 += nthreads * U) {
+    shortx8 v[U];
+    int dst[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u * nthreads;
+      dst[u] = -1;
+      if (c < total) {
+        const int key = c / per_key, rem = c - key * per_key;
+        const int g = rem / CPR, dc = rem - g * CPR;
+        const int tok = min(kv0 + key, last_tok);
+        const long row = (long)bt[tok / page] * page + tok % page;
+        v[u] = *reinterpret_cast<const shortx8 *>(src + (row * G + g) * D +
+                                                  dc * 8);
+        dst[u] = (g * key_stride + key) * KS + dc * 8;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (dst[u] >= 0) *reinterpret_cast<shortx8 *>(&kvbuf[dst[u]]) = v[u];
+  }
+}
 
 template <int D, int HPW>
 __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
@@ -418,15 +484,8 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
   const int kv_max = min(seq_len, past + min(q_len, (tile + 1) * MQ));
 
   auto stage = [&](const __hip_bfloat16 *__restrict__ src, int kv0) {
-    const int per_key = G * CPR;
-    for (int c = tid; c < MK * per_key; c += MWAVES * 64) {
-      const int key = c / per_key, rem = c - key * per_key;
-      const int g = rem / CPR, dc = rem - g * CPR;
-      const int tok = min(kv0 + key, seq_len - 1);
-      const long row = (long)bt[tok / page] * page + tok % page;
-      *reinterpret_cast<shortx8 *>(&kvbuf[(g * MK + key) * KS + dc * 8]) =
-          *reinterpret_cast<const shortx8 *>(src + (row * G + g) * D + dc * 8);
-    }
+    stage_tile<D>(kvbuf, src, bt, page, G, kv0, seq_len - 1, MK, MK, tid,
+                  MWAVES * 64);
   };
 
   for (int kv0 = 0; kv0 < kv_max; kv0 += MK) {
@@ -462,24 +521,35 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
     __syncthreads();
     stage(v_cache, kv0);   // K is done with; V lands while the heads talk
     // ---- mix + online softmax ----
+    // every raw plane is read once and feeds all heads of this wave
+    float svs[HPW][8];
+#pragma unroll
+    for (int hs = 0; hs < HPW; ++hs)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) svs[hs][e] = 0.f;
+#pragma unroll 2
+    for (int g2 = 0; g2 < H; ++g2) {
+      const float *row = sraw + (g2 * MQ + mi) * SR + mc * 8;
+      const floatx4 a0 = *reinterpret_cast<const floatx4 *>(row);
+      const floatx4 a1 = *reinterpret_cast<const floatx4 *>(row + 4);
+#pragma unroll
+      for (int hs = 0; hs < HPW; ++hs) {
+        const int h = min(wave + hs * MWAVES, H - 1);
+        const float t = tks[h * H + g2];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          svs[hs][e] += t * a0[e];
+          svs[hs][4 + e] += t * a1[e];
+        }
+      }
+    }
 #pragma unroll
     for (int hs = 0; hs < HPW; ++hs) {
       const int h = wave + hs * MWAVES;
       if (h < H) {
         float sv[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) sv[e] = 0.f;
-        for (int g2 = 0; g2 < H; ++g2) {
-          const float t = tks[h * H + g2];
-          const float *row = sraw + (g2 * MQ + mi) * SR + mc * 8;
-          const floatx4 a0 = *reinterpret_cast<const floatx4 *>(row);
-          const floatx4 a1 = *reinterpret_cast<const floatx4 *>(row + 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            sv[e] += t * a0[e];
-            sv[4 + e] += t * a1[e];
-          }
-        }
+        for (int e = 0; e < 8; ++e) sv[e] = svs[hs][e];
         float mx = -INFINITY;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -639,6 +709,269 @@ bool talking_attention_mfma(torch::Tensor &out, torch::Tensor &q,
     if (hpw == 1) GO(DV, 1);                                                \
     if (hpw == 2) GO(DV, 2);                                                \
     GO(DV, 4);                                                              \
+  }
+  GO_D(32)
+  GO_D(64)
+  GO_D(96)
+  GO_D(128)
+#undef GO_D
+#undef GO
+  return false;
+}
+
+// ------------------------------------------------------------------
+// bf16 decode-only batches (one new token per sequence). One workgroup =
+// (token, key split); the rep = H / G heads that share a kv head are the
+// MFMA rows, so a K/V tile is staged once and serves the whole group:
+//   stage K tile [G][32][D] -> LDS; S_grp = Q_grp K_g^T (16x16x32 MFMA)
+//   -> sraw[H][32]; stage V; mix + online softmax over the [H][32] plane
+//   (thread = head x key, stats in LDS); P -> pbuf (bf16);
+//   O_grp += P_grp V_g per (kv head, 16-column block) item, IT items per
+//   wave. Partials go through talking_merge_kernel when keys are split.
+namespace {
+
+constexpr int DSR = 33;   // sraw row stride (floats)
+
+template <int D, int IT>
+__global__ __launch_bounds__(MWAVES * 64) void talking_decode_mfma_kernel(
+    __hip_bfloat16 *__restrict__ out, float *__restrict__ part_acc,
+    float *__restrict__ part_ml, const __hip_bfloat16 *__restrict__ q,
+    long q_stride, const __hip_bfloat16 *__restrict__ k_cache,
+    const __hip_bfloat16 *__restrict__ v_cache,
+    const int *__restrict__ block_table, int bt_stride,
+    const int *__restrict__ seq_lens, int H, int G, int page, float scale,
+    const float *__restrict__ talk, const float *__restrict__ sink,
+    int splits) {
+  constexpr int KT = D / 32, NT = D / 16, KS = D + 8, CPR = D / 8;
+  extern __shared__ __attribute__((aligned(16))) char tk_lds[];
+  __hip_bfloat16 *kvbuf = reinterpret_cast<__hip_bfloat16 *>(tk_lds);
+  float *sraw = reinterpret_cast<float *>(tk_lds + (size_t)G * MK * KS * 2);
+  __hip_bfloat16 *pbuf = reinterpret_cast<__hip_bfloat16 *>(sraw + H * DSR + 3 - (H * DSR + 3) % 4);
+  float *alpha_s = reinterpret_cast<float *>(pbuf + H * PR);
+  float *mrun = alpha_s + H;
+  float *lrun = mrun + H;
+  float *tks = lrun + H;
+
+  const int t = blockIdx.x, sp = blockIdx.y;
+  const int total = seq_lens[t];            // keys 0 .. position
+  const int rep = H / G;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, lhi = lane >> 4;
+  const int *bt = block_table + (long)t * bt_stride;
+  const int tiles = (total + MK - 1) / MK;
+  const int tiles_per = (tiles + splits - 1) / splits;
+  const int j0 = sp * tiles_per * MK;
+  const int j1 = min(total, j0 + tiles_per * MK);
+
+  for (int d = tid; d < H * H; d += MWAVES * 64) tks[d] = talk[d];
+  for (int h = tid; h < H; h += MWAVES * 64) {
+    mrun[h] = -INFINITY;
+    lrun[h] = 0.f;
+  }
+  tk_f4 o_acc[IT];
+#pragma unroll
+  for (int ii = 0; ii < IT; ++ii) o_acc[ii] = tk_f4{0, 0, 0, 0};
+  const __hip_bfloat16 *qt = q + (long)t * q_stride;
+
+  auto stage = [&](const __hip_bfloat16 *__restrict__ src, int kv0) {
+    stage_tile<D>(kvbuf, src, bt, page, G, kv0, total - 1, MK, MK, tid,
+                  MWAVES * 64);
+  };
+
+  for (int kv0 = j0; kv0 < j1; kv0 += MK) {
+    stage(k_cache, kv0);
+    __syncthreads();
+    // ---- raw scores: item = (kv head, 16-key half) ----
+    for (int it = wave; it < 2 * G; it += MWAVES) {
+      const int g = it >> 1, f = it & 1;
+      tk_f4 s = tk_f4{0, 0, 0, 0};
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+        tk_bf8 a = tk_bf8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (l16 < rep)
+          a = *reinterpret_cast<const tk_bf8 *>(
+              qt + (g * rep + l16) * D + kt * 32 + lhi * 8);
+        const tk_bf8 bk = *reinterpret_cast<const tk_bf8 *>(
+            &kvbuf[(g * MK + f * 16 + l16) * KS + kt * 32 + lhi * 8]);
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bk, s, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (lhi * 4 + r < rep)
+          sraw[(g * rep + lhi * 4 + r) * DSR + f * 16 + l16] = s[r] * scale;
+    }
+    __syncthreads();
+    stage(v_cache, kv0);
+    // ---- mix + online softmax: thread = (head, key) ----
+    {
+      const int key = tid & 31;
+      const bool live = kv0 + key < j1;
+      for (int h = tid >> 5; h < H; h += MWAVES * 2) {
+        float sv = 0.f;
+#pragma unroll 4
+        for (int g2 = 0; g2 < H; ++g2)
+          sv += tks[h * H + g2] * sraw[g2 * DSR + key];
+        if (!live) sv = -INFINITY;
+        float mx = sv;
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1)
+          mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        const float m_old = mrun[h];
+        const float m_new = fmaxf(m_old, mx);
+        const float p = live ? expf(sv - m_new) : 0.f;
+        float psum = p;
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1)
+          psum += __shfl_xor(psum, off, 64);
+        const float alpha = m_old == -INFINITY ? 0.f : expf(m_old - m_new);
+        pbuf[h * PR + key] = __float2bfloat16(p);
+        if (key == 0) {
+          mrun[h] = m_new;
+          lrun[h] = lrun[h] * alpha + psum;
+          alpha_s[h] = alpha;
+        }
+      }
+    }
+    __syncthreads();
+    // ---- O += P V: item = (kv head, 16-column block) ----
+#pragma unroll
+    for (int ii = 0; ii < IT; ++ii) {
+      const int it = wave + ii * MWAVES;
+      if (it < G * NT) {
+        const int g = it / NT, nt = it - g * NT;
+        tk_bf8 pf = tk_bf8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (l16 < rep)
+          pf = *reinterpret_cast<const tk_bf8 *>(
+              &pbuf[(g * rep + l16) * PR + lhi * 8]);
+        const __hip_bfloat16 *vt =
+            kvbuf + (g * MK + lhi * 8) * KS + nt * 16 + l16;
+        tk_bf8 vf;
+        __hip_bfloat16 *ve = reinterpret_cast<__hip_bfloat16 *>(&vf);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ve[j] = vt[j * KS];
+        tk_f4 acc = o_acc[ii];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          acc[r] *= lhi * 4 + r < rep ? alpha_s[g * rep + lhi * 4 + r] : 0.f;
+        o_acc[ii] =
+            __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, acc, 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue ----
+  if (splits == 1) {
+    __syncthreads();
+    for (int h = tid; h < H; h += MWAVES * 64) {
+      float m = mrun[h], l = lrun[h], w = 1.f;
+      if (sink != nullptr) {
+        const float sk = sink[h];
+        const float M = fmaxf(m, sk);
+        w = m == -INFINITY ? 0.f : expf(m - M);
+        l = l * w + expf(sk - M);
+      }
+      alpha_s[h] = l > 0.f ? w / l : 0.f;
+    }
+    __syncthreads();
+  } else {
+    __syncthreads();
+    const long pbase = (long)t * splits + sp;
+    for (int h = tid; h < H; h += MWAVES * 64) {
+      part_ml[(pbase * H + h) * 2] = mrun[h];
+      part_ml[(pbase * H + h) * 2 + 1] = lrun[h];
+    }
+  }
+#pragma unroll
+  for (int ii = 0; ii < IT; ++ii) {
+    const int it = wave + ii * MWAVES;
+    if (it < G * NT) {
+      const int g = it / NT, nt = it - g * NT;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (lhi * 4 + r >= rep) continue;
+        const int h = g * rep + lhi * 4 + r;
+        const int col = h * D + nt * 16 + l16;
+        if (splits == 1)
+          out[(long)t * H * D + col] =
+              __float2bfloat16(o_acc[ii][r] * alpha_s[h]);
+        else
+          part_acc[((long)t * splits + sp) * H * D + col] = o_acc[ii][r];
+      }
+    }
+  }
+}
+
+template <int D, int IT>
+bool launch_talking_decode(torch::Tensor &out, torch::Tensor &q,
+                           torch::Tensor &k_cache, torch::Tensor &v_cache,
+                           torch::Tensor &block_table,
+                           torch::Tensor &seq_lens, double scale,
+                           torch::Tensor &talk, const float *sink, int splits,
+                           float *part_acc, float *part_ml, int H, int G,
+                           int page) {
+  const size_t sraw_f = ((size_t)H * DSR + 3) / 4 * 4;
+  const size_t lds = (size_t)G * MK * (D + 8) * 2 + sraw_f * 4 +
+                     (size_t)H * PR * 2 + (size_t)H * 3 * 4 +
+                     (size_t)H * H * 4;
+  if (lds > 160 * 1024) return false;
+  auto kern = talking_decode_mfma_kernel<D, IT>;
+  if (lds > 48 * 1024) {
+    static size_t granted = 0;
+    if (lds > granted) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+      }
+      granted = lds;
+    }
+  }
+  const int B = seq_lens.numel();
+  auto stream = at::cuda::getCurrentCUDAStream();
+  hipLaunchKernelGGL(kern, dim3(B, splits), dim3(MWAVES * 64), lds, stream,
+                     (__hip_bfloat16 *)out.data_ptr(), part_acc, part_ml,
+                     (const __hip_bfloat16 *)q.data_ptr(), (long)q.stride(0),
+                     (const __hip_bfloat16 *)k_cache.data_ptr(),
+                     (const __hip_bfloat16 *)v_cache.data_ptr(),
+                     block_table.data_ptr<int>(), (int)block_table.stride(0),
+                     seq_lens.data_ptr<int>(), H, G, page, (float)scale,
+                     talk.data_ptr<float>(), sink, splits);
+  HIP_CHECK_KERNEL();
+  return true;
+}
+
+}  // namespace
+
+bool talking_attention_decode_mfma(torch::Tensor &out, torch::Tensor &q,
+                                   torch::Tensor &k_cache,
+                                   torch::Tensor &v_cache,
+                                   torch::Tensor &block_table,
+                                   torch::Tensor &seq_lens, double scale,
+                                   torch::Tensor &talk, const float *sink,
+                                   int splits, float *part_acc,
+                                   float *part_ml) {
+  const int page = k_cache.size(1), G = k_cache.size(2), D = k_cache.size(3);
+  const int H = q.size(1) / D;
+  if (v_cache.size(3) != D || H / G > 16) return false;
+  if (reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 != 0 ||
+      (q.stride(0) * 2) % 16 != 0)
+    return false;
+  const int items = (G * (D / 16) + MWAVES - 1) / MWAVES;
+  if (items > 16) return false;
+  const int itc = items <= 2 ? 2 : items <= 4 ? 4 : items <= 8 ? 8 : 16;
+#define GO(DV, I)                                                          \
+  return launch_talking_decode<DV, I>(out, q, k_cache, v_cache,            \
+                                      block_table, seq_lens, scale, talk,  \
+                                      sink, splits, part_acc, part_ml, H,  \
+                                      G, page)
+#define GO_D(DV)                                                           \
+  if (D == DV) {                                                           \
+    if (itc == 2) GO(DV, 2);                                               \
+    if (itc == 4) GO(DV, 4);                                               \
+    if (itc == 8) GO(DV, 8);                                               \
+    GO(DV, 16);                                                            \
   }
   GO_D(32)
   GO_D(64)
