@@ -398,38 +398,84 @@ constexpr int MWAVES = 4;
 constexpr int SR = 36;   // sraw row stride (floats), 16 B aligned rows
 constexpr int PR = 40;   // pbuf row stride (bf16), 16 B aligned rows
 
-// One K or V tile [G][MK keys][D] from the paged cache into LDS rows of
-// KS elements; 16 B chunks, loads issued four at a time before their
-// stores so the global latency is paid once per batch.
+constexpr int VS = 40;   // V^T row stride (bf16): 32 keys + pad
+
+DEV_INLINE long cache_row(const int *__restrict__ bt, int page, int tok) {
+  return (long)bt[tok / page] * page + tok % page;
+}
+
+// K tile of MK keys, all kv heads, into LDS as [g][key][D + 8]: 16 B
+// chunks, a thread keeps the same (key, column chunk) for every kv head
+// (one page lookup per chunk), loads of two heads fly before their stores.
 template <int D>
-DEV_INLINE void stage_tile(__hip_bfloat16 *__restrict__ kvbuf,
-                           const __hip_bfloat16 *__restrict__ src,
-                           const int *__restrict__ bt, int page, int G,
-                           int kv0, int last_tok, int keys, int key_stride,
-                           int tid, int nthreads) {
-  constexpr int CPR = D / 8, KS = D + 8, U = 4;
-  const int per_key = G * CPR;
-  const int total = keys * per_key;
-  for (int c0 = tid; c0 < total; c0 += nthreads * U) {
+DEV_INLINE void stage_k_tile(__hip_bfloat16 *__restrict__ kvbuf,
+                             const __hip_bfloat16 *__restrict__ src,
+                             const int *__restrict__ bt, int page, int G,
+                             int kv0, int last_tok, int tid) {
+  constexpr int CPR = D / 8, KS = D + 8, NCH = MK * CPR;
+  constexpr int NTH = MWAVES * 64, UU = (NCH + NTH - 1) / NTH;
+  long off[UU];
+  int dst[UU];
+#pragma unroll
+  for (int u = 0; u < UU; ++u) {
+    const int c = tid + u * NTH;
+    const int key = c / CPR, dc = c - key * CPR;
+    dst[u] = c < NCH ? key * KS + dc * 8 : -1;
+    off[u] = cache_row(bt, page, min(kv0 + min(key, MK - 1), last_tok)) * G *
+                 D + dc * 8;
+  }
+  for (int g0 = 0; g0 < G; g0 += 2) {
+    shortx8 v[2][UU];
+#pragma unroll
+    for (int gg = 0; gg < 2; ++gg)
+#pragma unroll
+      for (int u = 0; u < UU; ++u)
+        if (g0 + gg < G && dst[u] >= 0)
+          v[gg][u] = *reinterpret_cast<const shortx8 *>(src + off[u] +
+                                                        (g0 + gg) * D);
+#pragma unroll
+    for (int gg = 0; gg < 2; ++gg)
+#pragma unroll
+      for (int u = 0; u < UU; ++u)
+        if (g0 + gg < G && dst[u] >= 0)
+          *reinterpret_cast<shortx8 *>(
+              &kvbuf[(g0 + gg) * MK * KS + dst[u]]) = v[gg][u];
+  }
+}
+
+// V tile transposed into LDS as [g][column][VS]: the P.V right operand
+// (8 consecutive keys of one column) is then one 16 B read, shared by
+// every head of the kv group. A thread owns one key (tid % 32) and
+// walks that key's 16 B chunks; the 2-byte stores of neighbouring lanes
+// fall into neighbouring keys of one column.
+template <int D>
+DEV_INLINE void stage_vt_tile(__hip_bfloat16 *__restrict__ kvbuf,
+                              const __hip_bfloat16 *__restrict__ src,
+                              const int *__restrict__ bt, int page, int G,
+                              int kv0, int last_tok, int tid) {
+  constexpr int CPR = D / 8, NTH = MWAVES * 64, SUBS = NTH / MK, U = 4;
+  const int key = tid & (MK - 1), sub = tid / MK;
+  const __hip_bfloat16 *rowp =
+      src + cache_row(bt, page, min(kv0 + key, last_tok)) * G * D;
+  const int nch = G * CPR;
+  for (int c0 = sub; c0 < nch; c0 += SUBS * U) {
     shortx8 v[U];
-    int dst[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int c = c0 + u * nthreads;
-      dst[u] = -1;
-      if (c < total) {
-        const int key = c / per_key, rem = c - key * per_key;
-        const int g = rem / CPR, dc = rem - g * CPR;
-        const int tok = min(kv0 + key, last_tok);
-        const long row = (long)bt[tok / page] * page + tok % page;
-        v[u] = *reinterpret_cast<const shortx8 *>(src + (row * G + g) * D +
-                                                  dc * 8);
-        dst[u] = (g * key_stride + key) * KS + dc * 8;
-      }
+      const int c = c0 + u * SUBS;
+      if (c < nch) v[u] = *reinterpret_cast<const shortx8 *>(rowp + c * 8);
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (dst[u] >= 0) *reinterpret_cast<shortx8 *>(&kvbuf[dst[u]]) = v[u];
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u * SUBS;
+      if (c < nch) {
+        // chunk c covers columns c*8 .. c*8+7 of the [G*D] row
+        const short *e = reinterpret_cast<const short *>(&v[u]);
+        short *dstp = reinterpret_cast<short *>(kvbuf) + (c * 8) * VS + key;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dstp[j * VS] = e[j];
+      }
+    }
   }
 }
 
@@ -442,10 +488,11 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
     const int *__restrict__ seq_lens, const int *__restrict__ qsl, int H,
     int G, int page, float scale, const float *__restrict__ talk,
     const float *__restrict__ sink) {
-  constexpr int KT = D / 32, NT = D / 16, KS = D + 8, CPR = D / 8;
+  constexpr int KT = D / 32, NT = D / 16, KS = D + 8;
   extern __shared__ __attribute__((aligned(16))) char tk_lds[];
   __hip_bfloat16 *kvbuf = reinterpret_cast<__hip_bfloat16 *>(tk_lds);
-  float *sraw = reinterpret_cast<float *>(tk_lds + (size_t)G * MK * KS * 2);
+  constexpr int KV_ELEMS = MK * KS > D * VS ? MK * KS : D * VS;
+  float *sraw = reinterpret_cast<float *>(tk_lds + (size_t)G * KV_ELEMS * 2);
   __hip_bfloat16 *pbuf =
       reinterpret_cast<__hip_bfloat16 *>(sraw + H * MQ * SR);
   float *alpha_s = reinterpret_cast<float *>(pbuf + H * MQ * PR);
@@ -483,13 +530,9 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
   const bool qrow_m_ok = qrow_m < q_len;
   const int kv_max = min(seq_len, past + min(q_len, (tile + 1) * MQ));
 
-  auto stage = [&](const __hip_bfloat16 *__restrict__ src, int kv0) {
-    stage_tile<D>(kvbuf, src, bt, page, G, kv0, seq_len - 1, MK, MK, tid,
-                  MWAVES * 64);
-  };
 
   for (int kv0 = 0; kv0 < kv_max; kv0 += MK) {
-    stage(k_cache, kv0);
+    stage_k_tile<D>(kvbuf, k_cache, bt, page, G, kv0, seq_len - 1, tid);
     __syncthreads();
     // ---- raw scores of this wave's heads ----
 #pragma unroll
@@ -519,8 +562,11 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
       }
     }
     __syncthreads();
-    stage(v_cache, kv0);   // K is done with; V lands while the heads talk
+    // K is done with; V^T lands while the heads talk
+    stage_vt_tile<D>(kvbuf, v_cache, bt, page, G, kv0, seq_len - 1, tid);
     // ---- mix + online softmax ----
+    const bool full_tile = kv0 + MK - 1 <= past + tile * MQ &&
+                           tile * MQ + MQ <= q_len;
     // every raw plane is read once and feeds all heads of this wave
     float svs[HPW][8];
 #pragma unroll
@@ -551,11 +597,17 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
 #pragma unroll
         for (int e = 0; e < 8; ++e) sv[e] = svs[hs][e];
         float mx = -INFINITY;
+        if (full_tile) {   // every key visible to every row: no mask lanes
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int kvp = kv0 + mc * 8 + e;
-          if (!qrow_m_ok || kvp > qpos_m || kvp >= seq_len) sv[e] = -INFINITY;
-          mx = fmaxf(mx, sv[e]);
+          for (int e = 0; e < 8; ++e) mx = fmaxf(mx, sv[e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int kvp = kv0 + mc * 8 + e;
+            if (!qrow_m_ok || kvp > qpos_m || kvp >= seq_len)
+              sv[e] = -INFINITY;
+            mx = fmaxf(mx, sv[e]);
+          }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
@@ -564,12 +616,12 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
         float pv[8], psum = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          pv[e] = sv[e] == -INFINITY ? 0.f : expf(sv[e] - m_new);
+          pv[e] = sv[e] == -INFINITY ? 0.f : __expf(sv[e] - m_new);
           psum += pv[e];
         }
         psum += __shfl_xor(psum, 1, 64);
         psum += __shfl_xor(psum, 2, 64);
-        const float alpha = m_old == -INFINITY ? 0.f : expf(m_old - m_new);
+        const float alpha = m_old == -INFINITY ? 0.f : __expf(m_old - m_new);
         l_run[hs] = l_run[hs] * alpha + psum;
         m_run[hs] = m_new;
         if (mc == 0) alpha_s[h * MQ + mi] = alpha;
@@ -589,13 +641,11 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
         for (int r = 0; r < 4; ++r) a4[r] = alpha_s[h * MQ + lhi * 4 + r];
         const tk_bf8 pf = *reinterpret_cast<const tk_bf8 *>(
             &pbuf[(h * MQ + l16) * PR + lhi * 8]);
-        const __hip_bfloat16 *vt = kvbuf + (g * MK + lhi * 8) * KS + l16;
+        const __hip_bfloat16 *vt = kvbuf + (g * D + l16) * VS + lhi * 8;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-          tk_bf8 vf;
-          __hip_bfloat16 *ve = reinterpret_cast<__hip_bfloat16 *>(&vf);
-#pragma unroll
-          for (int j = 0; j < 8; ++j) ve[j] = vt[j * KS + nt * 16];
+          const tk_bf8 vf =
+              *reinterpret_cast<const tk_bf8 *>(vt + nt * 16 * VS);
           tk_f4 acc = o_acc[hs][nt];
 #pragma unroll
           for (int r = 0; r < 4; ++r) acc[r] *= a4[r];
@@ -648,7 +698,8 @@ bool launch_talking_mfma(torch::Tensor &out, torch::Tensor &q,
                          torch::Tensor &query_start_loc, double scale,
                          torch::Tensor &talk, const float *sink,
                          long max_query_len, int H, int G, int page) {
-  const size_t lds = (size_t)G * MK * (D + 8) * 2 + (size_t)H * MQ * SR * 4 +
+  constexpr size_t kv_elems = MK * (D + 8) > D * VS ? MK * (D + 8) : D * VS;
+  const size_t lds = (size_t)G * kv_elems * 2 + (size_t)H * MQ * SR * 4 +
                      (size_t)H * MQ * PR * 2 + (size_t)H * MQ * 4 +
                      (size_t)H * H * 4;
   if (lds > 160 * 1024) return false;
@@ -742,11 +793,13 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_decode_mfma_kernel(
     const int *__restrict__ seq_lens, int H, int G, int page, float scale,
     const float *__restrict__ talk, const float *__restrict__ sink,
     int splits) {
-  constexpr int KT = D / 32, NT = D / 16, KS = D + 8, CPR = D / 8;
+  constexpr int KT = D / 32, NT = D / 16, KS = D + 8;
   extern __shared__ __attribute__((aligned(16))) char tk_lds[];
   __hip_bfloat16 *kvbuf = reinterpret_cast<__hip_bfloat16 *>(tk_lds);
-  float *sraw = reinterpret_cast<float *>(tk_lds + (size_t)G * MK * KS * 2);
-  __hip_bfloat16 *pbuf = reinterpret_cast<__hip_bfloat16 *>(sraw + H * DSR + 3 - (H * DSR + 3) % 4);
+  constexpr int KV_ELEMS = MK * KS > D * VS ? MK * KS : D * VS;
+  float *sraw = reinterpret_cast<float *>(tk_lds + (size_t)G * KV_ELEMS * 2);
+  __hip_bfloat16 *pbuf = reinterpret_cast<__hip_bfloat16 *>(
+      sraw + (H * DSR + 3) / 4 * 4);
   float *alpha_s = reinterpret_cast<float *>(pbuf + H * PR);
   float *mrun = alpha_s + H;
   float *lrun = mrun + H;
@@ -773,13 +826,9 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_decode_mfma_kernel(
   for (int ii = 0; ii < IT; ++ii) o_acc[ii] = tk_f4{0, 0, 0, 0};
   const __hip_bfloat16 *qt = q + (long)t * q_stride;
 
-  auto stage = [&](const __hip_bfloat16 *__restrict__ src, int kv0) {
-    stage_tile<D>(kvbuf, src, bt, page, G, kv0, total - 1, MK, MK, tid,
-                  MWAVES * 64);
-  };
 
   for (int kv0 = j0; kv0 < j1; kv0 += MK) {
-    stage(k_cache, kv0);
+    stage_k_tile<D>(kvbuf, k_cache, bt, page, G, kv0, total - 1, tid);
     __syncthreads();
     // ---- raw scores: item = (kv head, 16-key half) ----
     for (int it = wave; it < 2 * G; it += MWAVES) {
@@ -801,7 +850,7 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_decode_mfma_kernel(
           sraw[(g * rep + lhi * 4 + r) * DSR + f * 16 + l16] = s[r] * scale;
     }
     __syncthreads();
-    stage(v_cache, kv0);
+    stage_vt_tile<D>(kvbuf, v_cache, bt, page, G, kv0, total - 1, tid);
     // ---- mix + online softmax: thread = (head, key) ----
     {
       const int key = tid & 31;
@@ -818,12 +867,12 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_decode_mfma_kernel(
           mx = fmaxf(mx, __shfl_xor(mx, off, 64));
         const float m_old = mrun[h];
         const float m_new = fmaxf(m_old, mx);
-        const float p = live ? expf(sv - m_new) : 0.f;
+        const float p = live ? __expf(sv - m_new) : 0.f;
         float psum = p;
 #pragma unroll
         for (int off = 16; off > 0; off >>= 1)
           psum += __shfl_xor(psum, off, 64);
-        const float alpha = m_old == -INFINITY ? 0.f : expf(m_old - m_new);
+        const float alpha = m_old == -INFINITY ? 0.f : __expf(m_old - m_new);
         pbuf[h * PR + key] = __float2bfloat16(p);
         if (key == 0) {
           mrun[h] = m_new;
@@ -843,12 +892,8 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_decode_mfma_kernel(
         if (l16 < rep)
           pf = *reinterpret_cast<const tk_bf8 *>(
               &pbuf[(g * rep + l16) * PR + lhi * 8]);
-        const __hip_bfloat16 *vt =
-            kvbuf + (g * MK + lhi * 8) * KS + nt * 16 + l16;
-        tk_bf8 vf;
-        __hip_bfloat16 *ve = reinterpret_cast<__hip_bfloat16 *>(&vf);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) ve[j] = vt[j * KS];
+        const tk_bf8 vf = *reinterpret_cast<const tk_bf8 *>(
+            kvbuf + (g * D + nt * 16 + l16) * VS + lhi * 8);
         tk_f4 acc = o_acc[ii];
 #pragma unroll
         for (int r = 0; r < 4; ++r)
@@ -911,7 +956,8 @@ bool launch_talking_decode(torch::Tensor &out, torch::Tensor &q,
                            float *part_acc, float *part_ml, int H, int G,
                            int page) {
   const size_t sraw_f = ((size_t)H * DSR + 3) / 4 * 4;
-  const size_t lds = (size_t)G * MK * (D + 8) * 2 + sraw_f * 4 +
+  constexpr size_t kv_elems = MK * (D + 8) > D * VS ? MK * (D + 8) : D * VS;
+  const size_t lds = (size_t)G * kv_elems * 2 + sraw_f * 4 +
                      (size_t)H * PR * 2 + (size_t)H * 3 * 4 +
                      (size_t)H * H * 4;
   if (lds > 160 * 1024) return false;
