@@ -287,6 +287,9 @@ MODELS["hybrid-gdn-w2048"] = ("hybrid-GDN-w2048-8L",
                               hybrid_gdn_config(COMPARE_SIZES["w2048"]))
 MODELS["gukirax-w2048"] = ("Gukirax-w2048-8runs",
                            gukirax_config(COMPARE_SIZES["w2048"]))
+MODELS["sudevik-attn-w2048"] = (
+    "Sudevik-attn-w2048-8L",
+    sudevik_attention_config(COMPARE_SIZES["w2048"]))
 
 
 def mixer_compare(args):

@@ -418,7 +418,7 @@ def fused_moe_fp8(x: torch.Tensor, w13: torch.Tensor, w13_scale,
                    w13.view(torch.uint8), w13_scale.contiguous(),
                    sorted_ids, expert_blocks, n_post, None, n_pairs, topk,
                    gemm_m, False)
-    act = relu2(inter1) if activation == "relu2" else silu_and_mul(inter1)
+    act = silu_and_mul(inter1)
     actq, act_s = per_token_group_quant_fp8(act)
     pair_out = x.new_zeros(n_pairs, K)
     k.moe_gemm_fp8(pair_out, actq.view(torch.uint8), act_s,
@@ -552,7 +552,7 @@ def fused_moe_int4(x: torch.Tensor, w13_c, w13_sb, w2_c, w2_sb,
     k.moe_gemm_int4(inter1, x.contiguous(), w13_c, w13_sb, sorted_ids,
                     expert_blocks, n_post, None, n_pairs, topk, block_m,
                     False)
-    act = relu2(inter1) if activation == "relu2" else silu_and_mul(inter1)
+    act = silu_and_mul(inter1)
     pair_out = x.new_zeros(n_pairs, K)
     k.moe_gemm_int4(pair_out, act, w2_c, w2_sb, sorted_ids,
                     expert_blocks, n_post,
