@@ -479,6 +479,95 @@ DEV_INLINE void stage_vt_tile(__hip_bfloat16 *__restrict__ kvbuf,
   }
 }
 
+// Split forms of the two stagings for tiles small enough to ride in
+// registers (at most PF 16 B chunks per thread): the loads are issued
+// early and their stores come after independent work, so the global
+// latency hides behind the matrix and mix phases.
+constexpr int PF = 4;
+
+template <int D>
+DEV_INLINE bool tile_fits_regs(int G) {
+  constexpr int CPR = D / 8, NTH = MWAVES * 64;
+  constexpr int UU = (MK * CPR + NTH - 1) / NTH;
+  return G * UU <= PF && G * CPR <= PF * (NTH / MK);
+}
+
+template <int D>
+DEV_INLINE void k_tile_load(shortx8 (&v)[PF],
+                            const __hip_bfloat16 *__restrict__ src,
+                            const int *__restrict__ bt, int page, int G,
+                            int kv0, int last_tok, int tid) {
+  constexpr int CPR = D / 8, NCH = MK * CPR, NTH = MWAVES * 64;
+  constexpr int UU = (NCH + NTH - 1) / NTH;
+#pragma unroll
+  for (int u = 0; u < UU; ++u) {
+    const int c = tid + u * NTH;
+    const int key = c / CPR, dc = c - key * CPR;
+    if (c < NCH) {
+      const __hip_bfloat16 *rowp =
+          src + cache_row(bt, page, min(kv0 + key, last_tok)) * G * D + dc * 8;
+#pragma unroll
+      for (int g = 0; g < PF / UU; ++g)
+        if (g < G)
+          v[g * UU + u] = *reinterpret_cast<const shortx8 *>(rowp + g * D);
+    }
+  }
+}
+
+template <int D>
+DEV_INLINE void k_tile_store(__hip_bfloat16 *__restrict__ kvbuf,
+                             const shortx8 (&v)[PF], int G, int tid) {
+  constexpr int CPR = D / 8, KS = D + 8, NCH = MK * CPR, NTH = MWAVES * 64;
+  constexpr int UU = (NCH + NTH - 1) / NTH;
+#pragma unroll
+  for (int u = 0; u < UU; ++u) {
+    const int c = tid + u * NTH;
+    const int key = c / CPR, dc = c - key * CPR;
+    if (c < NCH) {
+#pragma unroll
+      for (int g = 0; g < PF / UU; ++g)
+        if (g < G)
+          *reinterpret_cast<shortx8 *>(
+              &kvbuf[(g * MK + key) * KS + dc * 8]) = v[g * UU + u];
+    }
+  }
+}
+
+template <int D>
+DEV_INLINE void vt_tile_load(shortx8 (&v)[PF],
+                             const __hip_bfloat16 *__restrict__ src,
+                             const int *__restrict__ bt, int page, int G,
+                             int kv0, int last_tok, int tid) {
+  constexpr int CPR = D / 8, SUBS = MWAVES * 64 / MK;
+  const int key = tid & (MK - 1), sub = tid / MK;
+  const __hip_bfloat16 *rowp =
+      src + cache_row(bt, page, min(kv0 + key, last_tok)) * G * D;
+  const int nch = G * CPR;
+#pragma unroll
+  for (int u = 0; u < PF; ++u) {
+    const int c = sub + u * SUBS;
+    if (c < nch) v[u] = *reinterpret_cast<const shortx8 *>(rowp + c * 8);
+  }
+}
+
+template <int D>
+DEV_INLINE void vt_tile_store(__hip_bfloat16 *__restrict__ kvbuf,
+                              const shortx8 (&v)[PF], int G, int tid) {
+  constexpr int CPR = D / 8, SUBS = MWAVES * 64 / MK;
+  const int key = tid & (MK - 1), sub = tid / MK;
+  const int nch = G * CPR;
+#pragma unroll
+  for (int u = 0; u < PF; ++u) {
+    const int c = sub + u * SUBS;
+    if (c < nch) {
+      const short *e = reinterpret_cast<const short *>(&v[u]);
+      short *dstp = reinterpret_cast<short *>(kvbuf) + (c * 8) * VS + key;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dstp[j * VS] = e[j];
+    }
+  }
+}
+
 template <int D, int HPW>
 __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
     __hip_bfloat16 *__restrict__ out, const __hip_bfloat16 *__restrict__ q,
@@ -531,8 +620,31 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
   const int kv_max = min(seq_len, past + min(q_len, (tile + 1) * MQ));
 
 
+  // the query fragments of this wave's heads stay in registers
+  tk_bf8 qf[HPW][KT];
+#pragma unroll
+  for (int hs = 0; hs < HPW; ++hs) {
+    const int h = min(wave + hs * MWAVES, H - 1);
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      qf[hs][kt] = tk_bf8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (qrow_a_ok)
+        qf[hs][kt] = *reinterpret_cast<const tk_bf8 *>(qa + h * D + kt * 32);
+    }
+  }
+  // small tiles travel through registers: K of the next tile is fetched
+  // under P V, V^T of this tile under Q K^T and the mix
+  const bool piped = tile_fits_regs<D>(G);
+  shortx8 kreg[PF], vreg[PF];
+  if (piped && kv_max > 0)
+    k_tile_load<D>(kreg, k_cache, bt, page, G, 0, seq_len - 1, tid);
   for (int kv0 = 0; kv0 < kv_max; kv0 += MK) {
-    stage_k_tile<D>(kvbuf, k_cache, bt, page, G, kv0, seq_len - 1, tid);
+    if (piped) {
+      k_tile_store<D>(kvbuf, kreg, G, tid);
+      vt_tile_load<D>(vreg, v_cache, bt, page, G, kv0, seq_len - 1, tid);
+    } else {
+      stage_k_tile<D>(kvbuf, k_cache, bt, page, G, kv0, seq_len - 1, tid);
+    }
     __syncthreads();
     // ---- raw scores of this wave's heads ----
 #pragma unroll
@@ -543,9 +655,7 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
         tk_f4 s0 = tk_f4{0, 0, 0, 0}, s1 = tk_f4{0, 0, 0, 0};
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
-          tk_bf8 a = tk_bf8{0, 0, 0, 0, 0, 0, 0, 0};
-          if (qrow_a_ok)
-            a = *reinterpret_cast<const tk_bf8 *>(qa + h * D + kt * 32);
+          const tk_bf8 a = qf[hs][kt];
           const tk_bf8 b0 = *reinterpret_cast<const tk_bf8 *>(
               &kvbuf[(g * MK + l16) * KS + kt * 32 + lhi * 8]);
           const tk_bf8 b1 = *reinterpret_cast<const tk_bf8 *>(
@@ -563,7 +673,8 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
     }
     __syncthreads();
     // K is done with; V^T lands while the heads talk
-    stage_vt_tile<D>(kvbuf, v_cache, bt, page, G, kv0, seq_len - 1, tid);
+    if (!piped)
+      stage_vt_tile<D>(kvbuf, v_cache, bt, page, G, kv0, seq_len - 1, tid);
     // ---- mix + online softmax ----
     const bool full_tile = kv0 + MK - 1 <= past + tile * MQ &&
                            tile * MQ + MQ <= q_len;
@@ -628,6 +739,12 @@ __global__ __launch_bounds__(MWAVES * 64) void talking_mfma_kernel(
         *reinterpret_cast<shortx8 *>(&pbuf[(h * MQ + mi) * PR + mc * 8]) =
             pack8<__hip_bfloat16>(pv);
       }
+    }
+    if (piped) {
+      vt_tile_store<D>(kvbuf, vreg, G, tid);
+      if (kv0 + MK < kv_max)
+        k_tile_load<D>(kreg, k_cache, bt, page, G, kv0 + MK, seq_len - 1,
+                       tid);
     }
     __syncthreads();
     // ---- O += P V ----
