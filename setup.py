@@ -7,12 +7,12 @@ repo snapshots without a site-packages install:
 
 * ``gllm_amd._kernels``      the kernel families of the other models
 * ``gllm_amd._kernels_seq``  the dtype-generic sequence-mixer kernels
-  (layer norm over an fp32 residual, windowed sink attention, varlen
-  gated delta rule) plus the grouped MoE GEMM, gated activations and
-  skinny GEMM that the linear / MoE layers dispatch to —
-  the only native code a Sudevik-style model needs, so a fresh
-  checkout can serve one after compiling eight files instead of
-  fifteen.
+  (layer norm over an fp32 residual, windowed sink attention,
+  talking-heads attention, varlen gated delta rule) plus the grouped
+  MoE GEMM, activations and skinny GEMM that the linear / MoE layers
+  dispatch to — the only native code a Sudevik- or Gukirax-style model
+  needs, so a fresh checkout can serve one after compiling nine files
+  instead of sixteen.
 
 ``GLLM_EXT=seq`` (or ``core``) restricts the build to one module.
 """
